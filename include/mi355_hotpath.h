@@ -639,6 +639,66 @@ int mi355_ar_status(void* comm, void* stream);
  * the next one in flight (overlap scheduling). */
 int mi355_ar_poll_status(void* comm);
 
+/* ---- a 32-bit residual stream whose sequences carry state across steps ---------------------------
+ * Models of the Seturax design (no counterpart in the reference).  The residual x is fp32 [tokens, hidden];
+ * `dtype` names the activation type T of everything the GEMMs around these kernels read and write.  The batch
+ * is described by tok_req / seg_start / seg_len (all three null: every token is its own one-token segment, the
+ * decode step) and `positions`; a sequence's state slot is req_to_state[req_pool_indices[b]].
+ *
+ * mi355_bigram_embedding: x[t] = table[id] * scale + bigram[(prev * mul_prev + id * mul_cur) mod buckets], row
+ *   `buckets` of `bigram` at position 0; prev is the token before t in its segment or, for a segment's first token,
+ *   prev_token[slot].
+ * mi355_layernorm_shift: h = (x - mean) / sqrt(var + eps) * weight (T, to h_out).  With `shift` given also
+ *   hs = h + (h_prev - h) * shift (to hs_out), h_prev being the previous token's h: zero at position 0, the fp32
+ *   row state[slot] for a segment's first token, recomputed from x[t - 1] otherwise; the fp32 h of every
+ *   segment's last token goes to h_last[b] (may be null).
+ * mi355_commit_sequence_state: after the step's last reader of the old state: state[l][slot] = h_last[l][b] for all
+ *   `layers`, and prev_token[slot] = the segment's last token id.
+ * mi355_gelu_tanh_and_mul: out[r][i] = gelu_tanh(gate[r][i]) * up[r][i], rows of gate / up `in_stride` apart.
+ * mi355_gated_residual_add: x[r][i] += sigmoid(g1[r][i] + b1[i]) * y1[r][i] (+ the same of g2, b2, y2 unless y2 is null). */
+int mi355_bigram_embedding(float* x, const int64_t* ids, const void* table, const void* bigram, const int32_t* prev_token,
+                           const int32_t* req_to_state, const int64_t* req_pool_indices, const int32_t* tok_req,
+                           const int32_t* seg_start, const int32_t* seg_len, const int64_t* positions, int64_t tokens,
+                           int64_t hidden, int64_t vocab, float scale, int64_t mul_prev, int64_t mul_cur, int64_t buckets,
+                           int dtype, void* stream);
+int mi355_layernorm_shift(void* h_out, void* hs_out, float* h_last, const float* x, const void* weight, const void* shift,
+                          const float* state, const int32_t* req_to_state, const int64_t* req_pool_indices,
+                          const int32_t* tok_req, const int32_t* seg_start, const int32_t* seg_len, const int64_t* positions,
+                          int64_t tokens, int64_t hidden, float eps, int dtype, void* stream);
+int mi355_commit_sequence_state(float* state, int32_t* prev_token, const float* h_last, const int64_t* ids,
+                                const int32_t* req_to_state, const int64_t* req_pool_indices, const int32_t* seg_start,
+                                const int32_t* seg_len, int64_t batch, int64_t layers, int64_t hidden, int64_t state_layer_stride,
+                                void* stream);
+int mi355_gelu_tanh_and_mul(void* out, const void* gate, const void* up, int64_t rows, int64_t d, int64_t in_stride, int dtype,
+                            void* stream);
+int mi355_gated_residual_add(float* x, const void* g1, const void* b1, const void* y1, const void* g2, const void* b2,
+                             const void* y2, int64_t rows, int64_t d, int64_t g_stride, int64_t y1_stride, int64_t y2_stride,
+                             int dtype, void* stream);
+
+/* ---- sliding-window attention over a latent KV cache with a softmax sink ---------------------------
+ * The cache row of a token is [c (rank) | k_r (rope_dim, rotated)].
+ * mi355_latent_norms_rope_write: from row t of the "a" projection, a[t] = [q latent (q_rank) | kv latent (rank) |
+ *   rope key (rope_dim) | ...]: cq[t] = RMSnorm(q latent) * q_weight, cache[loc[t]] = [RMSnorm(kv latent) * kv_weight |
+ *   rot(rope key)], the rotation pairing feature i with i + rot_dims / 2 at angle position * inv_freq[i] (fp32).
+ * mi355_latent_window_attention: out[t, h] = sum_j p(t, j) c[j] over the keys j of t's sequence with
+ *   0 <= position(t) - j < window, p = softmax with exp(sink[h]) added to the denominator of
+ *   (qa[t, h] . c[j] + rot(qr[t, h]) . k_r[j]) * scale; with `gate`, times sigmoid(gate[t * gate_stride + h]).
+ *   `blocks` lists runs (first token, count <= mi355_latent_window_attention_block_tokens(...)) of consecutive
+ *   tokens of one sequence, one workgroup each; null = one token per run and num_blocks = tokens.  The rows of the
+ *   new tokens must be in the cache already. */
+int mi355_latent_norms_rope_write(void* cq, void* cache, const void* a, const void* q_weight, const void* kv_weight,
+                                  const int64_t* positions, const int64_t* out_cache_loc, const float* inv_freq, int64_t tokens,
+                                  int64_t a_stride, int q_rank, int rank, int rope_dim, int rot_dims, int64_t num_slots, float eps,
+                                  int dtype, void* stream);
+int mi355_latent_window_attention_block_tokens(int heads, int rank, int rope_dim);
+int mi355_latent_window_attention(void* out, const void* qa, const void* qr, const void* cache, const void* gate,
+                                  const int32_t* req_to_token, const int64_t* req_pool_indices, const int32_t* tok_req,
+                                  const int64_t* positions, const int32_t* blocks, int64_t num_blocks, const float* sink,
+                                  const float* inv_freq, int64_t qa_token_stride, int64_t qa_head_stride, int64_t qr_token_stride,
+                                  int64_t qr_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t gate_stride,
+                                  int64_t req_to_token_stride, int heads, int rank, int rope_dim, int rot_dims, int window,
+                                  float scale, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -96,6 +96,14 @@ _SIGNATURES = {
     "mi355_argmax_chunked": (I, [P, P, L, L, L, P, L, P]),
     "mi355_softmax_temperature": (I, [P, P, L, L, L, P]),
     "mi355_top_k_top_p_min_p_sample": (I, [P, P, P, P, P, P, L, L, L, P]),
+    "mi355_bigram_embedding": (I, [P, P, P, P, P, P, P, P, P, P, P, L, L, L, F, L, L, L, I, P]),
+    "mi355_layernorm_shift": (I, [P, P, P, P, P, P, P, P, P, P, P, P, P, L, L, F, I, P]),
+    "mi355_commit_sequence_state": (I, [P, P, P, P, P, P, P, P, L, L, L, L, P]),
+    "mi355_gelu_tanh_and_mul": (I, [P, P, P, L, L, L, I, P]),
+    "mi355_gated_residual_add": (I, [P, P, P, P, P, P, P, L, L, L, L, L, I, P]),
+    "mi355_latent_norms_rope_write": (I, [P, P, P, P, P, P, P, P, L, L, I, I, I, I, L, F, I, P]),
+    "mi355_latent_window_attention_block_tokens": (I, [I, I, I]),
+    "mi355_latent_window_attention": (I, [P, P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, L, L, L, I, I, I, I, I, F, I, P]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

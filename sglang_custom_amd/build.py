@@ -13,7 +13,8 @@ LIB = os.path.join(HERE, "libmi355_hotpath.so")
 # variables set through mi355_debug_set) plus the bandwidth probes; used by tools/, never by the package
 LIB_DEV = os.path.join(HERE, "libmi355_hotpath_dev.so")
 SOURCES = ["elementwise.hip", "index_ops.hip", "attn_decode.hip", "attn_extend.hip", "gemm.hip",
-           "gemm_tiled.hip", "sampling.hip", "quant_fp8.hip", "allreduce.hip", "mla_proj.hip"]
+           "gemm_tiled.hip", "sampling.hip", "quant_fp8.hip", "allreduce.hip", "mla_proj.hip",
+           "stream_ops.hip", "attn_latent.hip"]
 DEV_SOURCES = ["debug_bw.hip"]
 HEADERS = [os.path.join(CSRC, "common.cuh"),
            os.path.join(os.path.dirname(HERE), "include", "mi355_hotpath.h"),
@@ -23,7 +24,10 @@ HEADERS = [os.path.join(CSRC, "common.cuh"),
 # form every such use costs a v_accvgpr_read/_write pair (hundreds per loop body in the attention
 # kernels), and no kernel needs more than the 256 registers the VGPR form can address.
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
-         "-Wno-unused-result", "-mllvm", "-amdgpu-mfma-vgpr-form"]
+         "-Wno-unused-result", "-mllvm", "-amdgpu-mfma-vgpr-form",
+         # no packed-fp32 instructions (v_pk_add/mul/fma_f32): the compiler forms them from ordinary float code by
+         # itself otherwise; the host pass does not know the feature and says so, harmlessly
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
 def _stale(target, deps):

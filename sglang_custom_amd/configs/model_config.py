@@ -17,6 +17,12 @@ class ModelConfig:
                  quantization: Optional[str] = None):
         c = dict(hf_config)
         self.hf_config = SimpleNamespace(**c)
+        self.architecture = c.get("architecture") or (c.get("architectures") or ["LlamaForCausalLM"])[0]
+        self.is_mla = False
+        self.needs_sequence_state = False
+        if self.architecture == "Seturax":
+            self._init_seturax(c, dtype, context_length, quantization)
+            return
         self.hidden_size = c["hidden_size"]
         self.num_hidden_layers = c["num_hidden_layers"]
         self.num_attention_heads = c["num_attention_heads"]
@@ -38,7 +44,7 @@ class ModelConfig:
         self.dtype = want
         self.is_encoder_decoder = False
         # multi-head latent attention (model_config.py:186-204): the cache holds one latent row per token
-        arch = (c.get("architectures") or [""])[0]
+        arch = self.architecture
         self.is_mla = arch in ("DeepseekV2ForCausalLM", "DeepseekV3ForCausalLM")
         if self.is_mla:
             self.head_dim = 256
@@ -48,6 +54,41 @@ class ModelConfig:
             self.v_head_dim = c["v_head_dim"]
             self.q_lora_rank = c.get("q_lora_rank")
             self.num_key_value_heads = 1
+
+    def _init_seturax(self, c: dict, dtype: str, context_length: Optional[int], quantization: Optional[str]) -> None:
+        """The Seturax design: config.json lists the layers one by one ("layers": [{"type", "mixer": {...}, "mlp":
+        {...} | null}]), with the widths under "width" / "vocab", the embedding's constants under "embedding" and the
+        norms' epsilon under "norm".  Every layer may have sizes of its own; what the pools and the attention backend
+        need as one number is the maximum over the layers."""
+        layers = c["layers"]
+        for i, spec in enumerate(layers):
+            if spec["type"] != "latent_attention":
+                raise ValueError(f"Seturax layer {i}: unknown mixer type {spec['type']!r}")
+            if spec.get("mlp") is not None and spec["mlp"].get("kind") != "dense":
+                raise ValueError(f"Seturax layer {i}: unknown feed-forward kind {spec['mlp'].get('kind')!r}")
+        self.layer_specs = layers
+        self.hidden_size = c["width"]
+        self.vocab_size = c["vocab"]
+        self.num_hidden_layers = len(layers)
+        self.num_attention_heads = max(s["mixer"]["heads"] for s in layers)
+        self.num_key_value_heads = 1
+        self.head_dim = max(s["mixer"]["kv_rank"] + s["mixer"]["rot_dim"] for s in layers)
+        self.v_head_dim = max(s["mixer"]["kv_rank"] for s in layers)
+        self.intermediate_size = max([s["mlp"]["ff"] for s in layers if s.get("mlp")] or [0])
+        self.rms_norm_eps = c["norm"]["eps"]
+        self.embedding_scale = c["embedding"]["scale"]
+        self.bigram = c["embedding"]["bigram"]
+        self.logit_scale = c.get("logit_scale", 1.0)
+        self.rope_theta = None
+        self.rope_scaling = None
+        self.tie_word_embeddings = False
+        self.max_position_embeddings = context_length or 131072     # the design fixes no longest sequence
+        self.context_len = self.max_position_embeddings
+        self.quantization = quantization
+        self.dtype = _DTYPES.get(dtype) or torch.bfloat16
+        self.is_encoder_decoder = False
+        self.needs_sequence_state = True     # previous token and previous normed rows travel from step to step
+        self.latent_kv = [(s["mixer"]["kv_rank"], s["mixer"]["rot_dim"]) for s in layers]
 
     @classmethod
     def from_path(cls, model_path: str, **kw) -> "ModelConfig":

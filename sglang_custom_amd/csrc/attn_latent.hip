@@ -1,0 +1,297 @@
+// Sliding-window attention over a latent KV cache, with a learned sink in the softmax denominator.
+//
+// The cache holds one row per token and layer: [ c (rank features) | k_r (rope features, already rotated) ].  In the
+// absorbed form every head h attends the same rows: score(t, j) = (qa[t,h] . c[j] + rot(qr[t,h]) . k_r[j]) * scale
+// with qa = q_nope W_uk[h], and the result per head is sum_j p(t, j) c[j] (the caller applies W_uv[h]).  Query at
+// position p sees key j iff 0 <= p - j < window.  softmax: p(t, j) = exp(s_j - m) / (sum_j exp(s_j - m) + exp(sink_h - m));
+// the sink has no value row, so the running (max, sum) pair simply starts at (sink_h, 1).
+//
+//   mi355_latent_norms_rope_write   the step before it: both latent RMS norms of the "a" projection's row, the
+//                                   rotation of the shared rope key and the write of the cache row
+//   mi355_latent_window_attention   prefill portions and decode steps alike: a workgroup takes a run of consecutive
+//                                   tokens of one sequence x a group of heads and walks the window's cache rows in
+//                                   LDS tiles; all arithmetic on scores, weights and sums is fp32
+#include "common.cuh"
+
+#include <algorithm>
+
+namespace mi355 {
+namespace {
+
+// ------------------------------------------------------------------------------------------ latent norms + rope + cache write
+// One workgroup per token.  a[t] = [ q latent (q_rank) | kv latent (rank) | rope key (dr) | ... ].
+template <typename T>
+__global__ __launch_bounds__(256) void latent_norms_rope_write_kernel(
+    T* __restrict__ cq, T* __restrict__ cache, const T* __restrict__ a, const T* __restrict__ wq, const T* __restrict__ wkv,
+    const int64_t* __restrict__ positions, const int64_t* __restrict__ loc, const float* __restrict__ inv_freq, int64_t a_stride,
+    int q_rank, int rank, int dr, int rot_dims, float eps) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const T* row = a + t * a_stride;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) {
+    const float v = to_f32(row[i]);
+    s += v * v;
+  }
+  const float inv_q = 1.0f / sqrtf(block_sum(s, red) / (float)q_rank + eps);
+  for (int i = threadIdx.x; i < q_rank; i += blockDim.x) cq[t * q_rank + i] = from_f32<T>(to_f32(row[i]) * inv_q * to_f32(wq[i]));
+  s = 0.f;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+    const float v = to_f32(row[q_rank + i]);
+    s += v * v;
+  }
+  const float inv_kv = 1.0f / sqrtf(block_sum(s, red) / (float)rank + eps);
+  T* dst = cache + loc[t] * (int64_t)(rank + dr);
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) dst[i] = from_f32<T>(to_f32(row[q_rank + i]) * inv_kv * to_f32(wkv[i]));
+  const T* kr = row + q_rank + rank;
+  const float pos = (float)positions[t];
+  const int half = rot_dims / 2;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float sn, cs;
+    sincosf(pos * inv_freq[i], &sn, &cs);
+    const float u = to_f32(kr[i]), v = to_f32(kr[i + half]);
+    dst[rank + i] = from_f32<T>(u * cs - v * sn);
+    dst[rank + i + half] = from_f32<T>(v * cs + u * sn);
+  }
+  for (int i = rot_dims + threadIdx.x; i < dr; i += blockDim.x) dst[rank + i] = kr[i];
+}
+
+// ------------------------------------------------------------------------------------------ attention
+struct LatentAttnParams {
+  const void* qa;        // [tokens, H, rank] through (qa_st, qa_sh)
+  const void* qr;        // unrotated rope part of q: element (t, h, i) at qr + t * qr_st + h * qr_sh + i
+  void* out;             // [tokens, H, rank] through (o_st, o_sh)
+  const void* cache;     // [slots, rank + dr]
+  const void* gate;      // per-(token, head) gate logits, or null
+  const int32_t* req_to_token;
+  const int64_t* req_pool_indices;
+  const int32_t* tok_req;     // null: token t belongs to sequence t
+  const int64_t* positions;
+  const int32_t* blocks;      // pairs (first token, count) of runs inside one sequence, or null: one token per run
+  const float* sink;          // [H]
+  const float* inv_freq;      // [rot_dims / 2]
+  int64_t qa_st, qa_sh, qr_st, qr_sh, o_st, o_sh, gate_st, rtt_stride;
+  int H, rank, dr, rot_dims, window, hg, kb, rows_cap;
+  float scale;
+};
+
+struct LatentAttnPlan {
+  int hg;        // heads per workgroup
+  int bq;        // tokens per workgroup
+  int kb;        // cache rows per LDS tile
+  size_t lds;
+};
+
+inline size_t latent_attn_lds(int m, int kb, int rank, int dr) {
+  const int rp = (rank + dr) | 1;
+  return sizeof(float) * ((size_t)m * rp + (size_t)kb * rp + (size_t)m * rank + (size_t)m * kb + 3 * (size_t)m) + sizeof(int) * kb;
+}
+
+inline LatentAttnPlan plan_latent_attn(int H, int rank, int dr) {
+  LatentAttnPlan p;
+  p.hg = std::min(H, 32);
+  p.bq = p.hg == H ? std::max(1, 32 / p.hg) : 1;
+  p.kb = 32;
+  const size_t budget = 150 * 1024;
+  while (latent_attn_lds(p.hg * p.bq, p.kb, rank, dr) > budget && p.kb > 8) p.kb /= 2;
+  while (latent_attn_lds(p.hg * p.bq, p.kb, rank, dr) > budget && p.bq > 1) p.bq -= 1;
+  while (latent_attn_lds(p.hg * p.bq, p.kb, rank, dr) > budget && p.hg > 1) p.hg = (p.hg + 1) / 2;
+  p.lds = latent_attn_lds(p.hg * p.bq, p.kb, rank, dr);
+  return p;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_window_attention_kernel(const LatentAttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) float smf[];
+  const int rank = p.rank, dr = p.dr, R = rank + dr, rp = R | 1, KB = p.kb;
+  int t0, n;
+  if (p.blocks) {
+    t0 = p.blocks[2 * blockIdx.x];
+    n = p.blocks[2 * blockIdx.x + 1];
+  } else {
+    t0 = blockIdx.x;
+    n = 1;
+  }
+  const int h0 = blockIdx.y * p.hg;
+  const int nh = min(p.hg, p.H - h0);
+  const int M = n * nh;
+  // LDS carve-up for the planned row count (the launch reserved bytes for rows_cap = hg * bq rows)
+  const int rows_cap = p.rows_cap;
+  float* Q = smf;                                // [rows_cap][rp]
+  float* K = Q + (size_t)rows_cap * rp;          // [KB][rp]
+  float* O = K + (size_t)KB * rp;                // [rows_cap][rank]
+  float* S = O + (size_t)rows_cap * rank;        // [rows_cap][KB]
+  float* mrow = S + (size_t)rows_cap * KB;
+  float* lrow = mrow + rows_cap;
+  float* arow = lrow + rows_cap;
+  int* kslot = reinterpret_cast<int*>(arow + rows_cap);
+
+  const T* qa = static_cast<const T*>(p.qa);
+  const T* qr = static_cast<const T*>(p.qr);
+  const T* cache = static_cast<const T*>(p.cache);
+  const int b = p.tok_req ? p.tok_req[t0] : t0;
+  const int64_t p0 = p.positions[t0];
+  const int32_t* table = p.req_to_token + p.req_pool_indices[b] * p.rtt_stride;
+  const int tid = threadIdx.x, nt = blockDim.x;
+
+  // ---- queries: absorbed part as is, rope part rotated by the token's position
+  for (int idx = tid; idx < M * rank; idx += nt) {
+    const int m = idx / rank, r = idx - m * rank;
+    const int ti = m / nh, hi = m - ti * nh;
+    Q[(size_t)m * rp + r] = to_f32(qa[(int64_t)(t0 + ti) * p.qa_st + (int64_t)(h0 + hi) * p.qa_sh + r]);
+  }
+  const int half = p.rot_dims / 2;
+  for (int idx = tid; idx < M * half; idx += nt) {
+    const int m = idx / half, i = idx - m * half;
+    const int ti = m / nh, hi = m - ti * nh;
+    const T* src = qr + (int64_t)(t0 + ti) * p.qr_st + (int64_t)(h0 + hi) * p.qr_sh;
+    float sn, cs;
+    sincosf((float)(p0 + ti) * p.inv_freq[i], &sn, &cs);
+    const float u = to_f32(src[i]), v = to_f32(src[i + half]);
+    Q[(size_t)m * rp + rank + i] = u * cs - v * sn;
+    Q[(size_t)m * rp + rank + i + half] = v * cs + u * sn;
+  }
+  const int tail = dr - p.rot_dims;
+  for (int idx = tid; idx < M * tail; idx += nt) {
+    const int m = idx / tail, i = p.rot_dims + (idx - m * tail);
+    const int ti = m / nh, hi = m - ti * nh;
+    Q[(size_t)m * rp + rank + i] = to_f32(qr[(int64_t)(t0 + ti) * p.qr_st + (int64_t)(h0 + hi) * p.qr_sh + i]);
+  }
+  for (int idx = tid; idx < M * rank; idx += nt) O[idx] = 0.f;
+  for (int m = tid; m < M; m += nt) {
+    mrow[m] = p.sink[h0 + (m % nh)];
+    lrow[m] = 1.0f;
+  }
+  __syncthreads();
+
+  const int64_t j_hi = p0 + n - 1;
+  const int64_t j_lo = max((int64_t)0, p0 - (int64_t)p.window + 1);
+  for (int64_t j0 = j_lo; j0 <= j_hi; j0 += KB) {
+    const int kn = (int)min((int64_t)KB, j_hi - j0 + 1);
+    for (int jj = tid; jj < kn; jj += nt) kslot[jj] = table[j0 + jj];
+    __syncthreads();
+    for (int idx = tid; idx < kn * R; idx += nt) {
+      const int jj = idx / R, r = idx - jj * R;
+      K[(size_t)jj * rp + r] = to_f32(cache[(int64_t)kslot[jj] * R + r]);
+    }
+    __syncthreads();
+    // ---- scores
+    for (int idx = tid; idx < M * KB; idx += nt) {
+      const int m = idx / KB, jj = idx - m * KB;
+      float s = -INFINITY;
+      if (jj < kn) {
+        const int64_t j = j0 + jj, pq = p0 + m / nh;
+        if (j <= pq && pq - j < p.window) {
+          const float* qrow = Q + (size_t)m * rp;
+          const float* krow = K + (size_t)jj * rp;
+          float acc = 0.f;
+          for (int r = 0; r < R; ++r) acc = fmaf(qrow[r], krow[r], acc);
+          s = acc * p.scale;
+        }
+      }
+      S[(size_t)m * KB + jj] = s;
+    }
+    __syncthreads();
+    // ---- running softmax per row
+    for (int m = tid; m < M; m += nt) {
+      float* srow = S + (size_t)m * KB;
+      const float mo = mrow[m];
+      float mx = mo;
+      for (int jj = 0; jj < kn; ++jj) mx = fmaxf(mx, srow[jj]);
+      const float alpha = expf(mo - mx);
+      float sum = 0.f;
+      for (int jj = 0; jj < kn; ++jj) {
+        const float e = expf(srow[jj] - mx);   // exp(-inf) = 0 for masked keys
+        srow[jj] = e;
+        sum += e;
+      }
+      mrow[m] = mx;
+      lrow[m] = lrow[m] * alpha + sum;
+      arow[m] = alpha;
+    }
+    __syncthreads();
+    // ---- weighted sum of the latent rows
+    for (int idx = tid; idx < M * rank; idx += nt) {
+      const int m = idx / rank, r = idx - m * rank;
+      const float* srow = S + (size_t)m * KB;
+      float acc = O[idx] * arow[m];
+      for (int jj = 0; jj < kn; ++jj) acc = fmaf(srow[jj], K[(size_t)jj * rp + r], acc);
+      O[idx] = acc;
+    }
+    __syncthreads();
+  }
+  T* out = static_cast<T*>(p.out);
+  const T* gate = static_cast<const T*>(p.gate);
+  for (int idx = tid; idx < M * rank; idx += nt) {
+    const int m = idx / rank, r = idx - m * rank;
+    const int ti = m / nh, hi = m - ti * nh;
+    float o = O[idx] / lrow[m];
+    if (gate) o *= 1.0f / (1.0f + expf(-to_f32(gate[(int64_t)(t0 + ti) * p.gate_st + h0 + hi])));
+    out[(int64_t)(t0 + ti) * p.o_st + (int64_t)(h0 + hi) * p.o_sh + r] = from_f32<T>(o);
+  }
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+int mi355_latent_norms_rope_write(void* cq, void* cache, const void* a, const void* q_weight, const void* kv_weight,
+                                  const int64_t* positions, const int64_t* out_cache_loc, const float* inv_freq, int64_t tokens,
+                                  int64_t a_stride, int q_rank, int rank, int rope_dim, int rot_dims, int64_t num_slots, float eps,
+                                  int dtype, void* stream) {
+  MI355_REQUIRE(cq && cache && a && q_weight && kv_weight && positions && out_cache_loc && inv_freq, MI355_ERR_INVALID,
+                "latent_norms_rope_write: null pointer");
+  MI355_REQUIRE(tokens >= 0 && q_rank > 0 && rank > 0 && rope_dim >= 0 && rot_dims >= 0 && rot_dims <= rope_dim && rot_dims % 2 == 0 &&
+                    a_stride >= (int64_t)q_rank + rank + rope_dim && num_slots > 0,
+                MI355_ERR_INVALID, "latent_norms_rope_write: bad shape");
+  if (tokens == 0) return MI355_OK;
+  MI355_DISPATCH_DTYPE(dtype, "latent_norms_rope_write", {
+    hipLaunchKernelGGL((latent_norms_rope_write_kernel<T>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, (T*)cq,
+                       (T*)cache, (const T*)a, (const T*)q_weight, (const T*)kv_weight, positions, out_cache_loc, inv_freq, a_stride,
+                       q_rank, rank, rope_dim, rot_dims, eps);
+  });
+  MI355_CHECK_LAUNCH("latent_norms_rope_write");
+  return MI355_OK;
+}
+
+int mi355_latent_window_attention_block_tokens(int heads, int rank, int rope_dim) {
+  if (heads <= 0 || rank <= 0 || rope_dim < 0) return 0;
+  const LatentAttnPlan pl = plan_latent_attn(heads, rank, rope_dim);
+  return pl.lds <= 160 * 1024 ? pl.bq : 0;
+}
+
+int mi355_latent_window_attention(void* out, const void* qa, const void* qr, const void* cache, const void* gate,
+                                  const int32_t* req_to_token, const int64_t* req_pool_indices, const int32_t* tok_req,
+                                  const int64_t* positions, const int32_t* blocks, int64_t num_blocks, const float* sink,
+                                  const float* inv_freq, int64_t qa_token_stride, int64_t qa_head_stride, int64_t qr_token_stride,
+                                  int64_t qr_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t gate_stride,
+                                  int64_t req_to_token_stride, int heads, int rank, int rope_dim, int rot_dims, int window,
+                                  float scale, int dtype, void* stream) {
+  MI355_REQUIRE(out && qa && cache && req_to_token && req_pool_indices && positions && sink, MI355_ERR_INVALID,
+                "latent_window_attention: null pointer");
+  MI355_REQUIRE(rope_dim == 0 || (qr && inv_freq), MI355_ERR_INVALID, "latent_window_attention: the rope part needs qr and inv_freq");
+  MI355_REQUIRE(heads > 0 && rank > 0 && rope_dim >= 0 && rot_dims >= 0 && rot_dims <= rope_dim && rot_dims % 2 == 0 && window > 0 &&
+                    num_blocks >= 0 && num_blocks < (1ll << 31),
+                MI355_ERR_INVALID, "latent_window_attention: bad shape");
+  if (num_blocks == 0) return MI355_OK;
+  const LatentAttnPlan pl = plan_latent_attn(heads, rank, rope_dim);
+  MI355_REQUIRE(pl.lds <= 160 * 1024, MI355_ERR_UNSUPPORTED, "latent_window_attention: rank %d + rope %d does not fit the LDS tile", rank,
+                rope_dim);
+  LatentAttnParams p;
+  p.qa = qa; p.qr = qr; p.out = out; p.cache = cache; p.gate = gate;
+  p.req_to_token = req_to_token; p.req_pool_indices = req_pool_indices; p.tok_req = tok_req; p.positions = positions;
+  p.blocks = blocks; p.sink = sink; p.inv_freq = inv_freq;
+  p.qa_st = qa_token_stride; p.qa_sh = qa_head_stride; p.qr_st = qr_token_stride; p.qr_sh = qr_head_stride;
+  p.o_st = out_token_stride; p.o_sh = out_head_stride; p.gate_st = gate_stride; p.rtt_stride = req_to_token_stride;
+  p.H = heads; p.rank = rank; p.dr = rope_dim; p.rot_dims = rot_dims; p.window = window; p.hg = pl.hg; p.kb = pl.kb; p.rows_cap = pl.hg * pl.bq;
+  p.scale = scale;
+  const dim3 grid((unsigned)num_blocks, (unsigned)((heads + pl.hg - 1) / pl.hg), 1);
+  MI355_DISPATCH_DTYPE(dtype, "latent_window_attention", {
+    auto kern = latent_window_attention_kernel<T>;
+    if (pl.lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds);
+    hipLaunchKernelGGL(kern, grid, dim3(256), pl.lds, (hipStream_t)stream, p);
+  });
+  MI355_CHECK_LAUNCH("latent_window_attention");
+  return MI355_OK;
+}

@@ -48,6 +48,7 @@ class ForwardMetadata:
     window_kv_indptr: Optional[torch.Tensor] = None
     window_kv_indices: Optional[torch.Tensor] = None
     window_num_kv_splits: int = 1
+    latent_blocks: Optional[dict] = None   # run length -> int32 [n, 2] token runs (forward_latent_window)
 
 
 class Mi355AttnBackend(AttentionBackend):
@@ -60,6 +61,9 @@ class Mi355AttnBackend(AttentionBackend):
         self.num_head = cfg.num_attention_heads // tp
         self.num_kv_head = max(1, cfg.num_key_value_heads // tp)
         self.is_mla = hasattr(model_runner.token_to_kv_pool, "kv_lora_rank")
+        # per-layer latent rows (LatentTokenToKVPool): served by forward_latent_window alone, whose only metadata is
+        # the list of token runs per workgroup
+        self.is_latent_window = hasattr(model_runner.token_to_kv_pool, "widths")
         self.kv_fp8 = getattr(model_runner.token_to_kv_pool, "dtype", None) == torch.float8_e4m3fn
         if self.is_mla:
             # what the split plan counts is workgroups per sequence, one per 16 query heads
@@ -131,6 +135,10 @@ class Mi355AttnBackend(AttentionBackend):
     def init_forward_metadata(self, forward_batch):
         ops = get_ops()
         bs = forward_batch.batch_size
+        if self.is_latent_window:
+            self.forward_metadata = ForwardMetadata()
+            self.forward_metadata.latent_blocks = {}
+            return
         if forward_batch.forward_mode.is_decode_or_idle():
             if forward_batch.seq_lens_cpu is not None and bs > 0:
                 max_len = int(forward_batch.seq_lens_cpu.max())
@@ -263,6 +271,40 @@ class Mi355AttnBackend(AttentionBackend):
             forward_batch.seq_lens, md.attn_logits, md.attn_lse, md.num_kv_splits,
             layer.scaling, layer.logit_cap, tickets=md.tickets, kv_chunk_keys=md.kv_chunk_keys)
         return o
+
+    # ---- sliding window over a latent cache, softmax sink ----
+    def _latent_blocks(self, forward_batch, bq: int) -> Optional[torch.Tensor]:
+        """int32 [n, 2] on the device: runs (first token, count <= bq) of consecutive tokens of one sequence, in token
+        order; None in a decode step (one token per run).  Built once per forward and run length."""
+        if forward_batch.forward_mode.is_decode():
+            return None
+        cache = self.forward_metadata.latent_blocks
+        if bq not in cache:
+            runs, t0 = [], 0
+            for n in forward_batch.extend_seq_lens_cpu:
+                full, rest = divmod(n, bq)
+                starts = torch.arange(t0, t0 + full * bq, bq, dtype=torch.int32)
+                runs.append(torch.stack([starts, torch.full_like(starts, bq)], 1))
+                if rest:
+                    runs.append(torch.tensor([[t0 + full * bq, rest]], dtype=torch.int32))
+                t0 += n
+            host = torch.cat(runs) if runs else torch.zeros((0, 2), dtype=torch.int32)
+            cache[bq] = host.contiguous().to(self.device, non_blocking=True)
+        return cache[bq]
+
+    def forward_latent_window(self, qa, qr, gate, layer, forward_batch, out):
+        """qa [T, H, rank] absorbed queries, qr [T, H, rope] unrotated, gate [T, H] logits or None -> out [T, H, rank].
+        The new tokens' rows are in the cache already (ops.latent_norms_rope_write); prefill portions, decode steps and
+        mixed batches are the same launch, told apart only by the list of token runs."""
+        ops = get_ops()
+        bq = ops.latent_window_attention_block_tokens(layer.tp_q_head_num, layer.kv_rank, layer.rope_dim)
+        if bq <= 0:
+            raise NotImplementedError(f"latent window attention: rank {layer.kv_rank} + rope {layer.rope_dim} is not served")
+        cache = forward_batch.token_to_kv_pool.get_key_buffer(layer.layer_id)
+        return ops.latent_window_attention(
+            qa, qr, cache, out, forward_batch.req_to_token_pool.req_to_token, forward_batch.req_pool_indices,
+            forward_batch.positions, layer.sink.data, layer.inv_freq, layer.rot_dims, layer.window, layer.scaling, gate=gate,
+            tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq))
 
     def _windowed(self, layer) -> bool:
         """triton_backend.py:656, 711: a layer with sliding_window_size > -1 attends the window lists."""

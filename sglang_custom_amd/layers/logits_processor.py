@@ -29,6 +29,8 @@ class LogitsProcessorOutput:
     input_token_logprobs: Optional[torch.Tensor] = None
     input_top_logprobs_val: Optional[list] = None
     input_top_logprobs_idx: Optional[list] = None
+    # fp32 logits of forward_batch.logits_rows, in that order
+    requested_logits: Optional[torch.Tensor] = None
 
 
 class LogitsProcessor(nn.Module):
@@ -58,7 +60,15 @@ class LogitsProcessor(nn.Module):
             if not logits.is_contiguous():   # a vocab-sliced view of padded logits
                 logits = logits.contiguous()
             ops.softcap_inplace(logits, self.final_logit_softcapping)
-        return LogitsProcessorOutput(next_token_logits=logits)
+        out = LogitsProcessorOutput(next_token_logits=logits)
+        rows = getattr(forward_batch, "logits_rows", None)
+        if rows is not None and rows.numel() > 0:
+            extra = self._get_logits(ops.embedding(rows, hidden_states.contiguous()), lm_head)
+            if self.final_logit_softcapping:
+                extra = extra.contiguous()
+                ops.softcap_inplace(extra, self.final_logit_softcapping)
+            out.requested_logits = extra
+        return out
 
     def _forward_with_input_logprobs(self, hidden_states, lm_head, fb) -> LogitsProcessorOutput:
         """The extend_return_logprob branch (logits_processor.py:274-420): logits of every prompt row from
@@ -119,6 +129,7 @@ class LogitsProcessor(nn.Module):
         else:
             logits = torch.matmul(x, w.T)
         if self.logit_scale is not None:
+            logits = logits.float()      # the scale is applied to the widened logits: one rounding, not two
             logits.mul_(self.logit_scale)
         if self.do_tensor_parallel_all_gather:
             logits = tensor_model_parallel_all_gather(logits)

@@ -180,3 +180,11 @@ def get_rope(head_size: int, rotary_dim: int, max_position: int, base: float,
         raise ValueError(f"RoPE scaling type {kind!r} is not supported by this backend")
     _ROPE_DICT[key] = rope
     return rope
+
+
+def rotate_half_inv_freq(base: float, dims: int) -> torch.Tensor:
+    """fp32 [dims / 2]: f_i = base^(-2 i / dims), the frequencies of a rotation that pairs feature i with
+    i + dims / 2.  For kernels that compute the angle position * f_i themselves, in fp32, instead of reading a
+    cos / sin table: nothing bounds the position."""
+    i = torch.arange(max(dims // 2, 1), dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / max(dims, 1)).to(torch.float32)

@@ -37,6 +37,7 @@ class Req:
         self.output_ids: List[int] = []
         self.sampling_params = sampling_params or SamplingParams(temperature=0)
         self.req_pool_idx: Optional[int] = None
+        self.state_slot: Optional[int] = None   # slot of the sequence-state pool, for models that carry state between steps
         # prefix reuse: slots of an already-cached prefix (empty without a prefix cache)
         self.prefix_indices = []
         self.fill_ids = self.origin_input_ids
@@ -124,6 +125,22 @@ class ScheduleBatch:
         return cls(reqs, req_to_token_pool, token_to_kv_pool_allocator, model_config,
                    req_to_token_pool.device)
 
+    @classmethod
+    def for_running(cls, reqs, req_to_token_pool, token_to_kv_pool_allocator, model_config, next_input_ids: torch.Tensor):
+        """A batch over requests that already hold their rows and KV (already_computed tokens each), ready for
+        prepare_for_decode() with next_input_ids as the step's tokens: what merge_batch / filter_batch leave behind
+        in the scheduler's running batch, built directly for a caller that picks the requests of a step itself."""
+        self = cls(list(reqs), req_to_token_pool, token_to_kv_pool_allocator, model_config, req_to_token_pool.device)
+        dev = self.device
+        lens = [r.already_computed for r in reqs]
+        self.req_pool_indices = torch.tensor([r.req_pool_idx for r in reqs], dtype=torch.int64).to(dev, non_blocking=True)
+        self.seq_lens = torch.tensor(lens, dtype=torch.int64).to(dev, non_blocking=True)
+        self.seq_lens_cpu_list = lens
+        self.seq_lens_sum = sum(lens)
+        self.output_ids = next_input_ids
+        self.sampling_info = SamplingBatchInfo.from_schedule_batch(self, model_config.vocab_size)
+        return self
+
     def batch_size(self) -> int:
         return len(self.reqs)
 
@@ -177,6 +194,8 @@ class ScheduleBatch:
                 req.extend_logprob_start_len = min(req.logprob_start_len - pre_len, req.extend_input_len, req.seqlen - 1)
             else:
                 req.extend_logprob_start_len = 0
+        if self.req_to_token_pool.state_pool is not None:
+            self.req_to_token_pool.take_state(reqs)
         self.top_logprobs_nums = [r.top_logprobs_num for r in reqs]
         self.extend_logprob_start_lens = [r.extend_logprob_start_len for r in reqs]
         self.extend_input_logprob_token_ids = None
@@ -339,4 +358,5 @@ class ScheduleBatch:
             slots = self.req_to_token_pool.req_to_token[r.req_pool_idx, :n].to(torch.int64)
             self.token_to_kv_pool_allocator.free(slots)
             self.req_to_token_pool.free(r.req_pool_idx)
+            self.req_to_token_pool.release_state(r)
             r.req_pool_idx = None

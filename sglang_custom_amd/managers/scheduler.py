@@ -44,6 +44,9 @@ CLIP_MAX_NEW_TOKENS = 4096
 class Scheduler:
     def __init__(self, model_runner, eos_token_id: Optional[int] = None, enable_radix_cache: bool = False):
         self.mr = model_runner
+        if enable_radix_cache and getattr(model_runner.req_to_token_pool, "state_pool", None) is not None:
+            # a cached prefix holds KV only; a sequence that starts behind one would lack the state its first token reads
+            raise ValueError("the prefix cache cannot serve a model whose sequences carry state between steps")
         self.page_size = getattr(model_runner.token_to_kv_pool_allocator, "page_size", 1)
         self.tree_cache = RadixCache(model_runner.req_to_token_pool, model_runner.token_to_kv_pool_allocator,
                                      disable=not enable_radix_cache, page_size=self.page_size)
@@ -245,6 +248,7 @@ class Scheduler:
             slots = pool.req_to_token[req.req_pool_idx, own_from:batch.seq_lens_cpu_list[idx]].to(torch.int64)
             alloc.free(slots)
             pool.free(req.req_pool_idx)
+            pool.release_state(req)
             if req.last_node is not None:
                 self.tree_cache.dec_lock_ref(req.last_node)
             self._make_room(len(order) * per_req)
@@ -287,6 +291,7 @@ class Scheduler:
             slots = pool.req_to_token[req.req_pool_idx, :seq_len].to(torch.int64)
             self.mr.token_to_kv_pool_allocator.free(slots)
             pool.free(req.req_pool_idx)
+        self.mr.req_to_token_pool.release_state(req)
         req.req_pool_idx = None
         req.last_node = None
         self.finished[req.rid] = req
@@ -387,6 +392,7 @@ class Scheduler:
             pool = self.mr.req_to_token_pool
             self.mr.token_to_kv_pool_allocator.free(pool.req_to_token[req.req_pool_idx, :held].to(torch.int64))
             pool.free(req.req_pool_idx)
+        self.mr.req_to_token_pool.release_state(req)
         req.req_pool_idx = None
         req.last_node = None
         self.finished[req.rid] = req

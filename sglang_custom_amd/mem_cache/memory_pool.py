@@ -24,6 +24,33 @@ class ReqToTokenPool:
         self.device = device
         self.req_to_token = torch.zeros((size, max_context_len), dtype=torch.int32, device=device)
         self.free_slots = list(range(size))
+        # models whose sequences carry state from step to step: the pool of state rows (SequenceStatePool) and the
+        # device map row of this table -> state slot, written when a request's row is (re)allocated
+        self.state_pool: Optional["SequenceStatePool"] = None
+        self.req_to_state: Optional[torch.Tensor] = None
+
+    def attach_state_pool(self, state_pool: "SequenceStatePool") -> None:
+        self.state_pool = state_pool
+        self.req_to_state = torch.zeros(self.size, dtype=torch.int32, device=self.device)
+
+    def take_state(self, reqs) -> None:
+        """Give every request of a new prefill batch that has none yet a state slot, and point the requests' rows of
+        this table at their slots (a request's row changes from one prefill portion to the next, its slot does not)."""
+        for r in reqs:
+            if r.state_slot is None:
+                r.state_slot = self.state_pool.alloc()
+                if r.state_slot is None:
+                    raise RuntimeError("out of sequence-state slots: raise max_running_requests")
+        self.bind_state([r.req_pool_idx for r in reqs], [r.state_slot for r in reqs])
+
+    def release_state(self, req) -> None:
+        if self.state_pool is not None and getattr(req, "state_slot", None) is not None:
+            self.state_pool.free(req.state_slot)
+            req.state_slot = None
+
+    def bind_state(self, req_rows: List[int], state_slots: List[int]) -> None:
+        rows = torch.tensor(req_rows, dtype=torch.int64).to(self.device, non_blocking=True)
+        self.req_to_state[rows] = torch.tensor(state_slots, dtype=torch.int32).to(self.device, non_blocking=True)
 
     def write(self, indices, values):
         self.req_to_token[indices] = values
@@ -46,6 +73,8 @@ class ReqToTokenPool:
 
     def clear(self):
         self.free_slots = list(range(self.size))
+        if self.state_pool is not None:
+            self.state_pool.clear()
 
 
 class MHATokenToKVPool:
@@ -169,3 +198,63 @@ class MLATokenToKVPool:
         T = loc.numel()
         row = torch.cat([cache_k_nope.reshape(T, 1, -1), cache_k_rope.reshape(T, 1, -1)], dim=-1)
         self.set_kv_buffer(layer, loc, row)
+
+
+class SequenceStatePool:
+    """State that a sequence carries from one step to the next, for models that have such (no counterpart in the
+    reference, whose models keep nothing but KV): per slot the last token id and, per layer, one fp32 row of the
+    model's width (the previous token's normed input of a token-shift layer).  A request holds one slot from its
+    first prefill portion until it finishes or is retracted; what a freed slot holds is never read again, because a
+    sequence's first token (position 0) takes no state.  Slot 0 is never handed out."""
+
+    def __init__(self, size: int, layer_num: int, hidden: int, device: str):
+        self.size = size
+        self.layer_num = layer_num
+        self.hidden = hidden
+        self.device = device
+        self.rows = torch.zeros((layer_num, size + 1, hidden), dtype=torch.float32, device=device)
+        self.prev_token = torch.zeros(size + 1, dtype=torch.int32, device=device)
+        self.free_slots = list(range(1, size + 1))
+
+    def available_size(self) -> int:
+        return len(self.free_slots)
+
+    def alloc(self) -> Optional[int]:
+        if not self.free_slots:
+            return None
+        return self.free_slots.pop(0)
+
+    def free(self, slot: int) -> None:
+        self.free_slots.append(slot)
+
+    def clear(self) -> None:
+        self.free_slots = list(range(1, self.size + 1))
+
+
+class LatentTokenToKVPool:
+    """Latent KV cache whose layers may differ in width: per layer one row [c (rank_l) | rotated rope key (rope_l)]
+    per token, [size + page_size, rank_l + rope_l]; slot 0 is the sink row of padded tokens, as in the other pools.
+    (MLATokenToKVPool is the special case of equal layers, kept for the DeepSeek kernels that assume one width.)"""
+
+    def __init__(self, size: int, page_size: int, dtype: torch.dtype, widths: List[Tuple[int, int]], device: str):
+        self.size = size
+        self.page_size = page_size
+        self.dtype = dtype
+        self.store_dtype = dtype
+        self.widths = list(widths)
+        self.layer_num = len(widths)
+        self.head_num = 1
+        self.device = device
+        self.kv_buffer = [torch.zeros((size + page_size, r + d), dtype=dtype, device=device) for r, d in widths]
+
+    def get_kv_size_bytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self.kv_buffer)
+
+    def get_key_buffer(self, layer_id: int) -> torch.Tensor:
+        return self.kv_buffer[layer_id]
+
+    def get_value_buffer(self, layer_id: int) -> torch.Tensor:
+        return self.kv_buffer[layer_id][..., : self.widths[layer_id][0]]
+
+    def get_kv_buffer(self, layer_id: int):
+        return self.get_key_buffer(layer_id), self.get_value_buffer(layer_id)

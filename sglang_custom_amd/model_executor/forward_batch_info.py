@@ -52,6 +52,28 @@ def clamp_position(seq_lens: torch.Tensor) -> torch.Tensor:
 
 
 @dataclasses.dataclass
+class SequenceStateBatch:
+    """One step's view of the per-sequence state (mem_cache.memory_pool.SequenceStatePool) for models whose sequences
+    carry state: how the flat token list splits into segments, where each sequence's state lives, and the staging rows
+    that the layers fill for the commit at the end of the step (the old state is read by every segment's first token,
+    so the new one is written only after the last layer)."""
+    pool: object
+    req_to_state: torch.Tensor
+    req_pool_indices: torch.Tensor
+    h_last: torch.Tensor                      # fp32 [layers, B, hidden]
+    tok_req: Optional[torch.Tensor] = None    # int32 [T]; None in a decode step (token b is sequence b)
+    seg_start: Optional[torch.Tensor] = None  # int32 [B]
+    seg_len: Optional[torch.Tensor] = None    # int32 [B]
+
+    def segments(self) -> dict:
+        return dict(tok_req=self.tok_req, seg_start=self.seg_start, seg_len=self.seg_len)
+
+    def commit(self, input_ids: torch.Tensor) -> None:
+        get_ops().commit_sequence_state(self.pool.rows, self.pool.prev_token, self.h_last, input_ids, self.req_to_state,
+                                        self.req_pool_indices, self.seg_start, self.seg_len)
+
+
+@dataclasses.dataclass
 class ForwardBatch:
     forward_mode: ForwardMode
     batch_size: int
@@ -77,6 +99,35 @@ class ForwardBatch:
     req_to_token_pool: object = None
     token_to_kv_pool: object = None
     attn_backend: object = None
+    # flat token indices whose logits the caller wants besides every sequence's last one (a replayed trace, scoring);
+    # LogitsProcessorOutput.requested_logits answers them
+    logits_rows: Optional[torch.Tensor] = None
+    seq_state: Optional[SequenceStateBatch] = None
+    _token_req_index: Optional[torch.Tensor] = None
+
+    def token_req_index(self) -> Optional[torch.Tensor]:
+        """int32 [T]: index in the batch of the sequence each token of an extend belongs to (None in a decode step)."""
+        if self.forward_mode.is_decode_or_idle():
+            return None
+        if self._token_req_index is None:
+            dev = self.extend_seq_lens.device
+            self._token_req_index = torch.repeat_interleave(
+                torch.arange(self.batch_size, dtype=torch.int32, device=dev), self.extend_seq_lens.to(torch.int64),
+                output_size=self.extend_num_tokens)
+        return self._token_req_index
+
+    def _init_seq_state(self, model_runner) -> None:
+        pool = getattr(self.req_to_token_pool, "state_pool", None)
+        if pool is None or self.forward_mode.is_idle():
+            return
+        h_last = torch.empty((pool.layer_num, self.batch_size, pool.hidden), dtype=torch.float32, device=model_runner.device)
+        st = SequenceStateBatch(pool=pool, req_to_state=self.req_to_token_pool.req_to_state,
+                                req_pool_indices=self.req_pool_indices, h_last=h_last)
+        if not self.forward_mode.is_decode():
+            st.tok_req = self.token_req_index()
+            st.seg_start = self.extend_start_loc
+            st.seg_len = self.extend_seq_lens
+        self.seq_state = st
 
     @classmethod
     def init_new(cls, batch, model_runner) -> "ForwardBatch":
@@ -115,4 +166,5 @@ class ForwardBatch:
             ids = getattr(batch, "extend_input_logprob_token_ids", None)
             if ids is not None:
                 ret.extend_input_logprob_token_ids_gpu = ids.to(device, non_blocking=True)
+        ret._init_seq_state(model_runner)
         return ret

@@ -14,8 +14,14 @@ from ..layers.logits_processor import LogitsProcessorOutput
 from ..layers.quantization.w8a8_fp8 import W8A8Fp8LinearMethod
 from ..layers.sampler import Sampler
 from ..mem_cache.allocator import PagedTokenToKVPoolAllocator, TokenToKVPoolAllocator
-from ..mem_cache.memory_pool import MHATokenToKVPool, MLATokenToKVPool, ReqToTokenPool
-from ..models.llama import LlamaForCausalLM
+from ..mem_cache.memory_pool import (
+    LatentTokenToKVPool,
+    MHATokenToKVPool,
+    MLATokenToKVPool,
+    ReqToTokenPool,
+    SequenceStatePool,
+)
+from ..models.registry import get_model_class
 from ..server_args import ServerArgs
 from .forward_batch_info import ForwardBatch
 
@@ -43,12 +49,8 @@ class ModelRunner:
             quant_factory = W8A8Fp8LinearMethod
         elif server_args.quantization is not None:
             raise ValueError(f"unsupported quantization {server_args.quantization!r}")
-        model_cls = LlamaForCausalLM
-        if getattr(model_config, "is_mla", False):
-            # registry lookup by config.architectures in the reference (model_loader/utils.py); two families here
-            from ..models.deepseek_v2 import DeepseekV2ForCausalLM
-
-            model_cls = DeepseekV2ForCausalLM
+        # registry lookup by the configuration's architecture name (model_loader/utils.py of the reference)
+        model_cls = get_model_class(getattr(model_config, "architecture", "LlamaForCausalLM"))
         self.model = model_cls(model_config, dtype=self.dtype, device=self.device,
                                quant_method_factory=quant_factory)
         if weights is not None:
@@ -62,7 +64,8 @@ class ModelRunner:
         self.attn_backend = (attn_backend_cls or Mi355AttnBackend)(self)
         self.graph_runner = None
         self.graph_capture_error = None
-        if not server_args.disable_cuda_graph and str(self.device).startswith("cuda"):
+        if (not server_args.disable_cuda_graph and str(self.device).startswith("cuda")
+                and getattr(self.model, "supports_hip_graph", True)):
             self.init_cuda_graphs()
 
     def init_cuda_graphs(self):
@@ -116,7 +119,10 @@ class ModelRunner:
             raise ValueError(f"kv_cache_dtype {kvd!r}: expected 'auto' or 'fp8_e4m3'")
         self.kv_cache_dtype = torch.float8_e4m3fn if kvd == "fp8_e4m3" else self.dtype
         mla = getattr(cfg, "is_mla", False)
-        if mla:
+        latent = getattr(cfg, "latent_kv", None)     # per-layer (rank, rope width) of a latent cache with unequal layers
+        if latent is not None:
+            cell = sum(r + d for r, d in latent) * torch.finfo(self.kv_cache_dtype).bits // 8
+        elif mla:
             # one latent row per token and layer (model_runner.py:950-957)
             cell = (cfg.kv_lora_rank + cfg.qk_rope_head_dim) * cfg.num_hidden_layers * torch.finfo(self.kv_cache_dtype).bits // 8
         else:
@@ -130,10 +136,18 @@ class ModelRunner:
         max_reqs = sa.max_running_requests or min(
             max(self.max_total_num_tokens // cfg.context_len * 512, 2048), 4096)
         self.req_to_token_pool = ReqToTokenPool(max_reqs, cfg.context_len + 4, self.device)
+        if getattr(self.model, "needs_sequence_state", False):
+            # one state slot per request that can be live at a time
+            self.req_to_token_pool.attach_state_pool(
+                SequenceStatePool(max_reqs, device=self.device, **self.model.sequence_state_spec()))
         page = max(1, int(getattr(sa, "page_size", 1) or 1))
         # whole pages only (model_runner.py:1101-1106 rounds the same way)
         self.max_total_num_tokens = self.max_total_num_tokens // page * page
-        if mla:
+        if latent is not None:
+            if self.kv_cache_dtype != self.dtype:
+                raise ValueError("a latent cache with per-layer widths is stored in the model dtype")
+            self.token_to_kv_pool = LatentTokenToKVPool(self.max_total_num_tokens, page, self.kv_cache_dtype, latent, self.device)
+        elif mla:
             # model_runner.py:1192-1206
             self.token_to_kv_pool = MLATokenToKVPool(
                 self.max_total_num_tokens, page, self.kv_cache_dtype, cfg.kv_lora_rank, cfg.qk_rope_head_dim,

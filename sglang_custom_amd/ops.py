@@ -1093,3 +1093,150 @@ def top_k_top_p_min_p_sample(probs: torch.Tensor, top_ks: Optional[torch.Tensor]
                                                  probs.shape[1], probs.stride(0), _stream(probs)),
           "top_k_top_p_min_p_sample")
     return ids
+
+
+# ------------------------------------------------------- fp32 residual stream with per-sequence state
+def _seg(tok_req, seg_start, seg_len):
+    assert (tok_req is None) == (seg_start is None) == (seg_len is None), "tok_req, seg_start and seg_len come together"
+    for t in (tok_req, seg_start, seg_len):
+        assert t is None or (t.dtype == torch.int32 and t.is_contiguous())
+    return _p(tok_req), _p(seg_start), _p(seg_len)
+
+
+def bigram_embedding(ids: torch.Tensor, table: torch.Tensor, bigram: torch.Tensor, prev_token: torch.Tensor,
+                     req_to_state: torch.Tensor, req_pool_indices: torch.Tensor, positions: torch.Tensor, scale: float,
+                     mul_prev: int, mul_cur: int, buckets: int, tok_req=None, seg_start=None, seg_len=None) -> torch.Tensor:
+    """fp32 [T, D]: table[id] * scale + bigram[(prev * mul_prev + id * mul_cur) % buckets] (row `buckets` at position 0);
+    prev comes from the batch or, for a segment's first token, from prev_token[state slot]."""
+    _gpu(ids, table, bigram, prev_token, req_to_state, req_pool_indices, positions)
+    assert ids.dtype == torch.int64 and positions.dtype == torch.int64 and req_pool_indices.dtype == torch.int64
+    assert prev_token.dtype == torch.int32 and req_to_state.dtype == torch.int32
+    assert table.is_contiguous() and bigram.is_contiguous() and table.dtype == bigram.dtype
+    assert bigram.shape == (buckets + 1, table.shape[1]) and ids.is_contiguous() and positions.is_contiguous()
+    T, D = ids.numel(), table.shape[1]
+    x = torch.empty((T, D), dtype=torch.float32, device=ids.device)
+    tr, ss, sl = _seg(tok_req, seg_start, seg_len)
+    check(_lib_().mi355_bigram_embedding(x.data_ptr(), ids.data_ptr(), table.data_ptr(), bigram.data_ptr(), prev_token.data_ptr(),
+                                         req_to_state.data_ptr(), req_pool_indices.data_ptr(), tr, ss, sl, positions.data_ptr(),
+                                         T, D, table.shape[0], float(scale), int(mul_prev), int(mul_cur), int(buckets),
+                                         _dt(table), _stream(ids)), "bigram_embedding")
+    return x
+
+
+def layernorm_shift(x: torch.Tensor, weight: torch.Tensor, eps: float, shift: Optional[torch.Tensor] = None, state=None,
+                    req_to_state=None, req_pool_indices=None, positions=None, h_last=None, tok_req=None, seg_start=None,
+                    seg_len=None):
+    """Weight-only layer norm of the fp32 rows x [T, D] -> h (weight's dtype).  With `shift` also the token-shifted rows
+    hs = h + (h_prev - h) * shift; returns h or (h, hs).  h_last [B, D] fp32 receives the h of every segment's last token."""
+    _gpu(x, weight, shift, state, req_to_state, req_pool_indices, positions, h_last)
+    assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and weight.is_contiguous()
+    T, D = x.shape
+    assert weight.numel() == D
+    h = torch.empty((T, D), dtype=weight.dtype, device=x.device)
+    hs = None
+    if shift is not None:
+        assert shift.dtype == weight.dtype and shift.numel() == D and shift.is_contiguous()
+        assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[-1] == D
+        assert req_to_state.dtype == torch.int32 and req_pool_indices.dtype == torch.int64 and positions.dtype == torch.int64
+        assert h_last is None or (h_last.dtype == torch.float32 and h_last.is_contiguous() and h_last.shape[-1] == D)
+        hs = torch.empty_like(h)
+    tr, ss, sl = _seg(tok_req, seg_start, seg_len)
+    check(_lib_().mi355_layernorm_shift(h.data_ptr(), _p(hs), _p(h_last) if shift is not None else None, x.data_ptr(),
+                                        weight.data_ptr(), _p(shift), _p(state), _p(req_to_state), _p(req_pool_indices),
+                                        tr, ss, sl, _p(positions), T, D, float(eps), _dt(weight), _stream(x)), "layernorm_shift")
+    return h if shift is None else (h, hs)
+
+
+def commit_sequence_state(state: torch.Tensor, prev_token: Optional[torch.Tensor], h_last: torch.Tensor, ids: torch.Tensor,
+                          req_to_state: torch.Tensor, req_pool_indices: torch.Tensor, seg_start=None, seg_len=None) -> None:
+    """state [L, slots, D] <- h_last [L, B, D] at every sequence's slot; prev_token[slot] <- the segment's last token id."""
+    _gpu(state, prev_token, h_last, ids, req_to_state, req_pool_indices)
+    L, B, D = h_last.shape
+    assert state.dim() == 3 and state.shape[0] == L and state.shape[2] == D and state.is_contiguous() and h_last.is_contiguous()
+    assert state.dtype == torch.float32 and h_last.dtype == torch.float32 and ids.dtype == torch.int64
+    assert req_pool_indices.numel() == B
+    _, ss, sl = _seg(seg_start, seg_start, seg_len)
+    check(_lib_().mi355_commit_sequence_state(state.data_ptr(), _p(prev_token), h_last.data_ptr(), ids.data_ptr(),
+                                              req_to_state.data_ptr(), req_pool_indices.data_ptr(), ss, sl, B, L, D,
+                                              state.stride(0), _stream(state)), "commit_sequence_state")
+
+
+def gelu_tanh_and_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """gelu_tanh(gate) * up for two [T, d] column blocks of one projection output (equal row strides)."""
+    _gpu(gate, up)
+    assert gate.dim() == 2 and gate.shape == up.shape and gate.dtype == up.dtype
+    assert gate.stride(1) == 1 and up.stride(1) == 1 and gate.stride(0) == up.stride(0)
+    out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    check(_lib_().mi355_gelu_tanh_and_mul(out.data_ptr(), gate.data_ptr(), up.data_ptr(), gate.shape[0], gate.shape[1],
+                                          gate.stride(0), _dt(gate), _stream(gate)), "gelu_tanh_and_mul")
+    return out
+
+
+def gated_residual_add(x: torch.Tensor, g1: torch.Tensor, b1: torch.Tensor, y1: torch.Tensor, g2=None, b2=None, y2=None) -> None:
+    """In place on the fp32 rows x: x += sigmoid(g1 + b1) * y1 (+ sigmoid(g2 + b2) * y2)."""
+    _gpu(x, g1, b1, y1, g2, b2, y2)
+    assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous()
+    T, D = x.shape
+    for t in (g1, y1, g2, y2):
+        assert t is None or (t.shape == (T, D) and t.stride(1) == 1 and t.dtype == g1.dtype)
+    assert b1.numel() == D and b1.dtype == g1.dtype and (g2 is None or g2.stride(0) == g1.stride(0))
+    check(_lib_().mi355_gated_residual_add(x.data_ptr(), g1.data_ptr(), b1.data_ptr(), y1.data_ptr(), _p(g2), _p(b2), _p(y2), T, D,
+                                           g1.stride(0), y1.stride(0), y2.stride(0) if y2 is not None else 0, _dt(g1),
+                                           _stream(x)), "gated_residual_add")
+
+
+# ------------------------------------------------------- windowed attention over a latent cache, softmax sink
+def latent_norms_rope_write(a: torch.Tensor, q_weight: torch.Tensor, kv_weight: torch.Tensor, positions: torch.Tensor,
+                            out_cache_loc: torch.Tensor, inv_freq: torch.Tensor, cache: torch.Tensor, q_rank: int, rank: int,
+                            rope_dim: int, rot_dims: int, eps: float) -> torch.Tensor:
+    """a [T, >= q_rank + rank + rope_dim]: returns cq = RMSnorm(a[:, :q_rank]) * q_weight and writes the cache rows
+    [RMSnorm(kv latent) * kv_weight | rot(rope key)] at out_cache_loc."""
+    _gpu(a, q_weight, kv_weight, positions, out_cache_loc, inv_freq, cache)
+    assert a.dim() == 2 and a.stride(1) == 1 and cache.is_contiguous() and cache.dtype == a.dtype
+    assert cache.shape[-1] == rank + rope_dim and q_weight.dtype == a.dtype == kv_weight.dtype
+    assert q_weight.numel() == q_rank and kv_weight.numel() == rank
+    assert inv_freq.dtype == torch.float32 and inv_freq.numel() >= rot_dims // 2
+    assert positions.dtype == torch.int64 and out_cache_loc.dtype == torch.int64
+    assert positions.is_contiguous() and out_cache_loc.is_contiguous()
+    T = a.shape[0]
+    cq = torch.empty((T, q_rank), dtype=a.dtype, device=a.device)
+    check(_lib_().mi355_latent_norms_rope_write(cq.data_ptr(), cache.data_ptr(), a.data_ptr(), q_weight.data_ptr(),
+                                                kv_weight.data_ptr(), positions.data_ptr(), out_cache_loc.data_ptr(),
+                                                inv_freq.data_ptr(), T, a.stride(0), q_rank, rank, rope_dim, rot_dims,
+                                                cache.shape[0], float(eps), _dt(a), _stream(a)), "latent_norms_rope_write")
+    return cq
+
+
+def latent_window_attention_block_tokens(heads: int, rank: int, rope_dim: int) -> int:
+    """Most consecutive tokens of one sequence that a workgroup of latent_window_attention takes (0: shape not served)."""
+    return int(_lib_().mi355_latent_window_attention_block_tokens(heads, rank, rope_dim))
+
+
+def latent_window_attention(qa: torch.Tensor, qr: torch.Tensor, cache: torch.Tensor, out: torch.Tensor, req_to_token: torch.Tensor,
+                            req_pool_indices: torch.Tensor, positions: torch.Tensor, sink: torch.Tensor, inv_freq: torch.Tensor,
+                            rot_dims: int, window: int, scale: float, gate: Optional[torch.Tensor] = None, tok_req=None,
+                            blocks=None) -> torch.Tensor:
+    """qa [T, H, rank] and out [T, H, rank] (any token / head strides), qr [T, H, rope_dim] unrotated, cache
+    [slots, rank + rope_dim], gate [T, H] logits (row-strided) or None, blocks int32 [n, 2] runs of tokens or None."""
+    _gpu(qa, qr, cache, out, req_to_token, req_pool_indices, positions, sink, inv_freq, gate, tok_req, blocks)
+    T, H, rank = qa.shape
+    rope_dim = cache.shape[-1] - rank
+    assert out.shape == qa.shape and qa.stride(2) == 1 and out.stride(2) == 1 and cache.is_contiguous()
+    assert qa.dtype == out.dtype == cache.dtype and sink.dtype == torch.float32 and sink.numel() == H and sink.is_contiguous()
+    assert req_to_token.dtype == torch.int32 and req_pool_indices.dtype == torch.int64 and positions.dtype == torch.int64
+    if rope_dim:
+        assert qr.shape == (T, H, rope_dim) and qr.stride(2) == 1 and qr.dtype == qa.dtype and inv_freq.dtype == torch.float32
+    assert gate is None or (gate.shape == (T, H) and gate.stride(1) == 1 and gate.dtype == qa.dtype)
+    assert tok_req is None or (tok_req.dtype == torch.int32 and tok_req.numel() == T)
+    if blocks is not None:
+        assert blocks.dtype == torch.int32 and blocks.dim() == 2 and blocks.shape[1] == 2 and blocks.is_contiguous()
+        nb = blocks.shape[0]
+    else:
+        nb = T
+    check(_lib_().mi355_latent_window_attention(
+        out.data_ptr(), qa.data_ptr(), _p(qr) if rope_dim else None, cache.data_ptr(), _p(gate), req_to_token.data_ptr(),
+        req_pool_indices.data_ptr(), _p(tok_req), positions.data_ptr(), _p(blocks), nb, sink.data_ptr(), _p(inv_freq),
+        qa.stride(0), qa.stride(1), qr.stride(0) if rope_dim else 0, qr.stride(1) if rope_dim else 0, out.stride(0), out.stride(1),
+        gate.stride(0) if gate is not None else 0, req_to_token.stride(0), H, rank, rope_dim, rot_dims, int(window), float(scale),
+        _dt(qa), _stream(qa)), "latent_window_attention")
+    return out

@@ -185,3 +185,137 @@ def mla_prefill_assemble_supported(nope, rope, vd, rank, dtype):
     """The one-launch prefill glue is a GPU kernel only: the double declines and the model takes rotary_emb + the
     copies + set_kv_buffer, which is what the oracle restates."""
     return False
+
+
+# ------------------------------------------------------- fp32 residual stream with per-sequence state
+# Restatements of the kernels' contracts (include/mi355_hotpath.h) token by token; they share nothing with the
+# whole-sequence functions of oracle/seturax_ref.py that the tests compare against.
+def _segments(T, tok_req, seg_start, seg_len):
+    """(b, first, last) per token."""
+    if tok_req is None:
+        return [(t, True, True) for t in range(T)]
+    out = []
+    for t in range(T):
+        b = int(tok_req[t])
+        s, n = int(seg_start[b]), int(seg_len[b])
+        out.append((b, t == s, t == s + n - 1))
+    return out
+
+
+def bigram_embedding(ids, table, bigram, prev_token, req_to_state, req_pool_indices, positions, scale, mul_prev, mul_cur,
+                     buckets, tok_req=None, seg_start=None, seg_len=None):
+    T = ids.numel()
+    x = torch.empty((T, table.shape[1]), dtype=torch.float32)
+    for t, (b, first, _) in enumerate(_segments(T, tok_req, seg_start, seg_len)):
+        tok = int(ids[t])
+        if int(positions[t]) == 0:
+            row = buckets
+        else:
+            prev = int(prev_token[int(req_to_state[int(req_pool_indices[b])])]) if first else int(ids[t - 1])
+            row = (prev * mul_prev + tok * mul_cur) % buckets
+        x[t] = table[tok].float() * scale + bigram[row].float()
+    return x
+
+
+def _ln(row, w, eps):
+    mu = row.mean()
+    var = ((row - mu) ** 2).mean()
+    return (row - mu) / torch.sqrt(var + eps) * w.float()
+
+
+def layernorm_shift(x, weight, eps, shift=None, state=None, req_to_state=None, req_pool_indices=None, positions=None,
+                    h_last=None, tok_req=None, seg_start=None, seg_len=None):
+    T, D = x.shape
+    h32 = torch.stack([_ln(x[t], weight, eps) for t in range(T)]) if T else x.new_zeros((0, D))
+    if shift is None:
+        return h32.to(weight.dtype)
+    hs = torch.empty_like(h32)
+    for t, (b, first, last) in enumerate(_segments(T, tok_req, seg_start, seg_len)):
+        if int(positions[t]) == 0:
+            prev = torch.zeros(D)
+        elif first:
+            prev = state[int(req_to_state[int(req_pool_indices[b])])]
+        else:
+            prev = h32[t - 1]
+        hs[t] = h32[t] + (prev - h32[t]) * shift.float()
+        if last and h_last is not None:
+            h_last[b] = h32[t]
+    return h32.to(weight.dtype), hs.to(weight.dtype)
+
+
+def commit_sequence_state(state, prev_token, h_last, ids, req_to_state, req_pool_indices, seg_start=None, seg_len=None):
+    L, B, D = h_last.shape
+    for b in range(B):
+        slot = int(req_to_state[int(req_pool_indices[b])])
+        state[:, slot] = h_last[:, b]
+        last = b if seg_start is None else int(seg_start[b]) + int(seg_len[b]) - 1
+        if prev_token is not None:
+            prev_token[slot] = int(ids[last])
+
+
+def gelu_tanh_and_mul(gate, up):
+    z = gate.float()
+    g = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
+    return (g * up.float()).to(gate.dtype)
+
+
+def gated_residual_add(x, g1, b1, y1, g2=None, b2=None, y2=None):
+    add = torch.sigmoid(g1.float() + b1.float()) * y1.float()
+    if y2 is not None:
+        add = add + torch.sigmoid(g2.float() + b2.float()) * y2.float()
+    x.add_(add)
+
+
+def _rot(v, pos, inv_freq, rot_dims):
+    half = rot_dims // 2
+    ang = float(pos) * inv_freq[:half].float()
+    c, s = torch.cos(ang), torch.sin(ang)
+    u, w = v[..., :half].float(), v[..., half:rot_dims].float()
+    return torch.cat([u * c - w * s, w * c + u * s, v[..., rot_dims:].float()], -1)
+
+
+def latent_norms_rope_write(a, q_weight, kv_weight, positions, out_cache_loc, inv_freq, cache, q_rank, rank, rope_dim,
+                            rot_dims, eps):
+    T = a.shape[0]
+    cq = torch.empty((T, q_rank), dtype=a.dtype)
+    for t in range(T):
+        row = a[t].float()
+        q = row[:q_rank]
+        cq[t] = (q / torch.sqrt((q * q).mean() + eps) * q_weight.float()).to(a.dtype)
+        c = row[q_rank: q_rank + rank]
+        c = c / torch.sqrt((c * c).mean() + eps) * kv_weight.float()
+        kr = _rot(row[q_rank + rank: q_rank + rank + rope_dim], positions[t], inv_freq, rot_dims)
+        cache[int(out_cache_loc[t])] = torch.cat([c, kr]).to(cache.dtype)
+    return cq
+
+
+def latent_window_attention_block_tokens(heads, rank, rope_dim):
+    return 3
+
+
+def latent_window_attention(qa, qr, cache, out, req_to_token, req_pool_indices, positions, sink, inv_freq, rot_dims, window,
+                            scale, gate=None, tok_req=None, blocks=None):
+    T, H, rank = qa.shape
+    covered = torch.zeros(T, dtype=torch.bool)
+    runs = [(t, 1) for t in range(T)] if blocks is None else [(int(a), int(n)) for a, n in blocks.tolist()]
+    for t0, n in runs:
+        for t in range(t0, t0 + n):
+            assert not covered[t]
+            covered[t] = True
+            b = t if tok_req is None else int(tok_req[t])
+            assert blocks is None or int(tok_req[t0]) == b, "a run crosses two sequences"
+            p = int(positions[t])
+            lo = max(0, p - window + 1)
+            slots = req_to_token[int(req_pool_indices[b]), lo: p + 1].long()
+            rows = cache[slots].float()                                  # [n_keys, rank + rope]
+            q = torch.cat([qa[t].float(), _rot(qr[t], p, inv_freq, rot_dims)], -1)   # [H, rank + rope]
+            s = (q @ rows.T) * scale                                     # [H, n_keys]
+            m = torch.maximum(s.max(-1).values, sink.float())
+            e = torch.exp(s - m[:, None])
+            pr = e / (e.sum(-1) + torch.exp(sink.float() - m))[:, None]
+            o = pr @ rows[:, :rank]
+            if gate is not None:
+                o = o * torch.sigmoid(gate[t].float())[:, None]
+            out[t] = o.to(out.dtype)
+    assert bool(covered.all()), "the runs do not cover every token"
+    return out
