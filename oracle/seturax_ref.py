@@ -164,3 +164,20 @@ def greedy(cfg: dict, weights: Dict[str, torch.Tensor], prompt: List[int], n: in
     for _ in range(n):
         toks.append(int(forward(cfg, weights, toks, dtype)[-1].argmax()))
     return toks[len(prompt):]
+
+
+def absorbed_window_attention(qa: torch.Tensor, qr: torch.Tensor, c: torch.Tensor, kr: torch.Tensor, sink: torch.Tensor,
+                              scale: float, window: int, base: float, dims: int, gate: Optional[torch.Tensor] = None,
+                              first_position: int = 0) -> torch.Tensor:
+    """The attention of latent_attention() with the key expansion folded into the query: qa [T, H, rank] multiplies
+    the latent rows c [n, rank] directly, qr [T, H, dr] is the unrotated rope part, kr [n, dr] the ROTATED shared rope
+    key of every cached position 0..n-1; the T queries sit at positions first_position .. first_position + T - 1
+    (= n - 1).  Returns sum_j p_j c_j per head [T, H, rank], times sigmoid(gate [T, H]) if given."""
+    T, n = qa.shape[0], c.shape[0]
+    pos = torch.arange(first_position, first_position + T)
+    q_rot = rotate_half(qr, pos, base, dims)
+    scores = (torch.einsum("ihr,jr->hij", qa, c) + torch.einsum("ihd,jd->hij", q_rot, kr)) * scale
+    mask = window_mask(n, window)[first_position: first_position + T]
+    pr = sink_softmax(scores, mask, sink)
+    o = torch.einsum("hij,jr->ihr", pr, c)
+    return o if gate is None else o * torch.sigmoid(gate)[..., None]

@@ -1,0 +1,172 @@
+"""Seturax on the CPU: the package's host side (configuration, weight stacking, model wiring, ScheduleBatch /
+ForwardBatch, the KV / request / state pools, TraceReplayer, Scheduler) runs with the CPU checker ops (tests/cpu_ops.py)
+and every logit is compared with the plain whole-sequence implementation in oracle/seturax_ref.py.  The HIP kernels
+have their own file (test_seturax_gpu.py); here the arithmetic is the checker's, the bookkeeping is the product's."""
+import pytest
+import torch
+
+import seturax_util as su
+from oracle import seturax_ref as ref
+
+TOL = 2e-5
+
+
+@pytest.fixture(autouse=True)
+def _cpu_backend():
+    import cpu_ops
+    from sglang_custom_amd import ops_backend
+    from sglang_custom_amd.distributed import parallel_state
+
+    prev = ops_backend._backend
+    ops_backend.set_ops_backend(cpu_ops)
+    parallel_state.init_distributed_environment(1, 0)
+    yield
+    ops_backend.set_ops_backend(prev)
+
+
+@pytest.fixture(scope="module")
+def model():
+    cfg = su.make_config()
+    return cfg, su.make_weights(cfg, seed=3)
+
+
+def test_oracle_pieces_agree_with_each_other():
+    """The absorbed form of the oracle's attention equals its expanded form (keys and values from the latent)."""
+    torch.manual_seed(0)
+    cfg = su.make_config()
+    w = {k: v.double() for k, v in su.make_weights(cfg, 1).items()}
+    mx, T, D = cfg["layers"][0]["mixer"], 11, cfg["width"]
+    h = torch.randn(T, D, dtype=torch.float64)
+    full = ref.latent_attention(h, w, "l0.mix.", mx, 1e-5)
+    H, dn, dr, dv, rank = mx["heads"], mx["dim"], mx["rot_dim"], mx["vdim"], mx["kv_rank"]
+    q = (ref.rms_norm(h @ w["l0.mix.dq"].T, w["l0.mix.dq.norm"], 1e-5) @ w["l0.mix.uq"].T).reshape(T, H, dn + dr)
+    kv = h @ w["l0.mix.dkv"].T
+    c = ref.rms_norm(kv[:, :rank], w["l0.mix.dkv.norm"], 1e-5)
+    kr = ref.rotate_half(kv[:, None, rank:], torch.arange(T), mx["rot"]["base"], mx["rot"]["dims"])[:, 0]
+    qa = torch.einsum("thd,hdr->thr", q[..., :dn], w["l0.mix.uk"].view(H, dn, rank))
+    o = ref.absorbed_window_attention(qa, q[..., dn:], c, kr, w["l0.mix.sink"], mx["scale"], mx["mask"]["size"],
+                                      mx["rot"]["base"], mx["rot"]["dims"], gate=h @ w["l0.mix.g"].T)
+    out = torch.einsum("thr,hvr->thv", o, w["l0.mix.uv"].view(H, dv, rank)).reshape(T, H * dv) @ w["l0.mix.o"].T
+    assert (out - full).abs().max() < 1e-10
+
+
+def test_whole_prompt_then_token_by_token(model):
+    cfg, w = model
+    prompts = su.random_prompts(cfg, [23])
+    mr = su.build_runner(cfg, w)
+    su.replay_and_compare(mr, cfg, w, prompts, [[("r0", 23)]], TOL)
+    su.replay_and_compare(mr, cfg, w, prompts, [[("r0", 1)] for _ in range(23)], TOL)
+    su.replay_and_compare(mr, cfg, w, prompts, [[("r0", 9)]] + [[("r0", 1)] for _ in range(14)], TOL)
+    assert su.pools_are_whole(mr)
+
+
+@pytest.mark.parametrize("sizes", [[2, 2, 2, 3, 5, 2, 7, 1, 1, 2], [1, 4, 4, 4, 4, 4, 4, 2], [25, 2]])
+def test_portions_of_any_size(model, sizes):
+    cfg, w = model
+    n = sum(sizes)
+    prompts = su.random_prompts(cfg, [n], seed=5)
+    mr = su.build_runner(cfg, w)
+    su.replay_and_compare(mr, cfg, w, prompts, [[("r0", k)] for k in sizes], TOL)
+    assert su.pools_are_whole(mr)
+
+
+@pytest.mark.parametrize("page_size", [1, 4])
+def test_mixed_batches_reuse_slots_and_pages(model, page_size):
+    """Unequal requests side by side -- portions beside single tokens, a request that sits a step out, requests that end
+    while others go on -- in a pool so small that KV slots, request rows and state slots are all handed out again."""
+    cfg, w = model
+    prompts = su.random_prompts(cfg, [17, 9, 1, 12, 20, 6], seed=7)
+    sched = [[("r0", 5), ("r1", 2)], [("r0", 1), ("r1", 7), ("r2", 1)], [("r0", 4), ("r3", 3)], [("r3", 1)],
+             [("r0", 1), ("r3", 1)], [("r0", 6), ("r3", 7), ("r4", 2)], [("r4", 1), ("r5", 1)], [("r4", 1), ("r5", 1)],
+             [("r4", 9), ("r5", 4)], [("r4", 1)], [("r4", 6)]]
+    mr = su.build_runner(cfg, w, max_total_tokens=48, max_running_requests=3, page_size=page_size)
+    su.replay_and_compare(mr, cfg, w, prompts, sched, TOL)
+    assert su.pools_are_whole(mr)
+    # the same again on the used pools: stale rows, stale state
+    su.replay_and_compare(mr, cfg, w, prompts, sched, TOL)
+    assert su.pools_are_whole(mr)
+
+
+def test_equal_and_unit_sizes():
+    """Sizes that a model may happen to make equal or 1: one head, rope width equal to the head width, value width
+    equal to the rank, window 1 and a window longer than any prompt, width equal to the vocabulary."""
+    layers = [(su.mixer(1, 4, 4, 8, 8, 8, 1), 8), (su.mixer(4, 2, 2, 2, 2, 2, 1000), None)]
+    cfg = su.make_config(width=16, vocab=16, layers=layers, buckets=1, mul_prev=1, mul_cur=1, scale=1.0, logit_scale=1.0)
+    w = su.make_weights(cfg, seed=11)
+    prompts = su.random_prompts(cfg, [14, 5], seed=1)
+    mr = su.build_runner(cfg, w, max_total_tokens=32)
+    su.replay_and_compare(mr, cfg, w, prompts, [[("r0", 3), ("r1", 1)], [("r0", 1), ("r1", 1)], [("r0", 10), ("r1", 3)]], TOL)
+
+
+def test_state_is_what_the_next_step_reads(model):
+    """Cutting a prompt must hand over exactly the previous token and the previous normed rows: a corrupted state row
+    or token changes the next portion's logits, and position 0 reads neither."""
+    cfg, w = model
+    from sglang_custom_amd.managers.trace_replay import TraceReplayer
+
+    prompts = su.random_prompts(cfg, [8], seed=2)["r0"]
+    mr = su.build_runner(cfg, w)
+    pool = mr.req_to_token_pool.state_pool
+    pool.rows.fill_(123.0)          # what an earlier owner may have left: a first token must not see it
+    pool.prev_token.fill_(5)
+    rp = TraceReplayer(mr)
+    want = ref.forward(cfg, w, prompts)
+    assert su.rel_err(rp.step([dict(id="a", tokens=prompts[:4], want=[0, 1, 2, 3])]), want[:4]) < TOL
+    slot = rp.live["a"].state_slot
+    assert int(pool.prev_token[slot]) == prompts[3]
+    good = pool.rows[:, slot].clone()
+    pool.rows[1, slot] += 1.0
+    assert su.rel_err(rp.step([dict(id="a", tokens=prompts[4:5], want=[0])]), want[4:5]) > 1e-3
+    rp.finish("a")
+    # the same with the token alone corrupted
+    rp.step([dict(id="b", tokens=prompts[:4], want=[])])
+    slot = rp.live["b"].state_slot
+    assert torch.equal(pool.rows[:, slot], good)
+    pool.prev_token[slot] = (prompts[3] + 1) % cfg["vocab"]
+    assert su.rel_err(rp.step([dict(id="b", tokens=prompts[4:5], want=[0])], ["b"]), want[4:5]) > 1e-3
+    assert su.pools_are_whole(mr)
+
+
+@pytest.mark.parametrize("chunk,mixed", [(None, False), (6, False), (6, True)])
+def test_greedy_generation_through_the_scheduler(model, chunk, mixed):
+    """The package's own entry point: requests queued at the Scheduler, prompts chunked by its policy, decode batches
+    (and decode tokens riding prefill batches) formed by it, tokens picked by the Sampler."""
+    from sglang_custom_amd.managers.schedule_batch import Req
+    from sglang_custom_amd.managers.scheduler import Scheduler
+    from sglang_custom_amd.sampling.sampling_params import SamplingParams
+
+    cfg, w = model
+    prompts = su.random_prompts(cfg, [11, 3, 7, 15, 1], seed=9)
+    mr = su.build_runner(cfg, w, max_total_tokens=96, max_running_requests=3, chunked_prefill_size=chunk, enable_mixed_chunk=mixed)
+    sch = Scheduler(mr)
+    for k, p in prompts.items():
+        sch.add_request(Req(k, p, SamplingParams(temperature=0, max_new_tokens=6)))
+    done = sch.run_until_done()
+    for k, p in prompts.items():
+        assert done[k].output_ids == ref.greedy(cfg, w, p, 6), k
+    assert su.pools_are_whole(mr)
+    if chunk:
+        assert sch.num_prefill_batches > 3
+
+
+def test_prefix_cache_is_refused(model):
+    from sglang_custom_amd.managers.scheduler import Scheduler
+
+    cfg, w = model
+    with pytest.raises(ValueError):
+        Scheduler(su.build_runner(cfg, w), enable_radix_cache=True)
+
+
+def test_configuration_is_read_not_assumed():
+    from sglang_custom_amd.configs.model_config import ModelConfig
+    from sglang_custom_amd.models.registry import get_model_class
+
+    cfg = su.make_config()
+    mc = ModelConfig(cfg, dtype="float32")
+    assert mc.architecture == "Seturax" and get_model_class(mc.architecture).__name__ == "SeturaxForCausalLM"
+    assert mc.latent_kv == [(10, 4), (24, 8), (16, 2)] and mc.num_attention_heads == 3 and mc.needs_sequence_state
+    bad = su.make_config()
+    bad["layers"][1]["type"] = "something_else"
+    with pytest.raises(ValueError):
+        ModelConfig(bad)
+    assert get_model_class("LlamaForCausalLM").__name__ == "LlamaForCausalLM"
