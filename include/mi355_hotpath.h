@@ -685,19 +685,22 @@ int mi355_gated_residual_add(float* x, const void* g1, const void* b1, const voi
  *   (qa[t, h] . c[j] + rot(qr[t, h]) . k_r[j]) * scale; with `gate`, times sigmoid(gate[t * gate_stride + h]).
  *   `blocks` lists runs (first token, count <= mi355_latent_window_attention_block_tokens(...)) of consecutive
  *   tokens of one sequence, one workgroup each; null = one token per run and num_blocks = tokens.  The rows of the
- *   new tokens must be in the cache already. */
+ *   new tokens must be in the cache already.  16-bit dtypes with rank <= 512 run on the matrix cores (64 query rows per
+ *   workgroup); there, with blocks == null, num_splits > 1 cuts every token's keys into that many ranges, one workgroup
+ *   each, whose partial results (split_scratch: num_splits * tokens * heads * (rank + 2) floats) a second launch merges.
+ *   fp32 and wider ranks run a vector-ALU kernel (num_splits = 1). */
 int mi355_latent_norms_rope_write(void* cq, void* cache, const void* a, const void* q_weight, const void* kv_weight,
                                   const int64_t* positions, const int64_t* out_cache_loc, const float* inv_freq, int64_t tokens,
                                   int64_t a_stride, int q_rank, int rank, int rope_dim, int rot_dims, int64_t num_slots, float eps,
                                   int dtype, void* stream);
-int mi355_latent_window_attention_block_tokens(int heads, int rank, int rope_dim);
+int mi355_latent_window_attention_block_tokens(int heads, int rank, int rope_dim, int dtype);
 int mi355_latent_window_attention(void* out, const void* qa, const void* qr, const void* cache, const void* gate,
                                   const int32_t* req_to_token, const int64_t* req_pool_indices, const int32_t* tok_req,
                                   const int64_t* positions, const int32_t* blocks, int64_t num_blocks, const float* sink,
                                   const float* inv_freq, int64_t qa_token_stride, int64_t qa_head_stride, int64_t qr_token_stride,
                                   int64_t qr_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t gate_stride,
                                   int64_t req_to_token_stride, int heads, int rank, int rope_dim, int rot_dims, int window,
-                                  float scale, int dtype, void* stream);
+                                  float scale, int num_splits, float* split_scratch, int64_t tokens, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

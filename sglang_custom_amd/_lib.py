@@ -102,8 +102,8 @@ _SIGNATURES = {
     "mi355_gelu_tanh_and_mul": (I, [P, P, P, L, L, L, I, P]),
     "mi355_gated_residual_add": (I, [P, P, P, P, P, P, P, L, L, L, L, L, I, P]),
     "mi355_latent_norms_rope_write": (I, [P, P, P, P, P, P, P, P, L, L, I, I, I, I, L, F, I, P]),
-    "mi355_latent_window_attention_block_tokens": (I, [I, I, I]),
-    "mi355_latent_window_attention": (I, [P, P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, L, L, L, I, I, I, I, I, F, I, P]),
+    "mi355_latent_window_attention_block_tokens": (I, [I, I, I, I]),
+    "mi355_latent_window_attention": (I, [P, P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, L, L, L, I, I, I, I, I, F, I, P, L, I, P]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

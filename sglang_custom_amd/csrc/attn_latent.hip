@@ -73,6 +73,13 @@ struct LatentAttnParams {
   int64_t qa_st, qa_sh, qr_st, qr_sh, o_st, o_sh, gate_st, rtt_stride;
   int H, rank, dr, rot_dims, window, hg, kb, rows_cap;
   float scale;
+  // matrix-core kernel only: the keys of a run cut into nsplit ranges, one workgroup each; unnormalised partial
+  // sums, maxima and denominators go to part_o / part_m / part_l ([nsplit][tokens][H][...]) for the merge kernel
+  int nsplit;
+  int64_t tokens;
+  float* part_o;
+  float* part_m;
+  float* part_l;
 };
 
 struct LatentAttnPlan {
@@ -231,6 +238,271 @@ __global__ __launch_bounds__(256) void latent_window_attention_kernel(const Late
   }
 }
 
+
+// ------------------------------------------------------------------------------------------ matrix-core kernel (16-bit)
+// 64 query rows (tokens x heads) per workgroup, 16 per wave; cache rows in LDS tiles of 32 keys shared by the four
+// waves.  S = Q K^T on v_mfma_f32_16x16x32 (both operands read as 16-byte fragments of their LDS rows, so the number
+// of 32-wide chunks is a run-time loop), softmax on the fp32 accumulators (a row's 32 scores sit in 16 lanes x 2
+// registers), P rounded to T and passed through LDS into the A layout of v_mfma_f32_16x16x16, whose B operand -- the
+// value part of the same K tile -- comes from a transposed LDS read.  NRT = 16-column tiles of the value part kept
+// in registers (compile time: 4 accumulators each).
+constexpr int LM_KB = 32;
+constexpr int LM_ROWS = 64;
+constexpr int LM_PLD = LM_KB + 8;
+
+inline int lm_ld(int rank, int dr) { return ((rank + dr + 31) & ~31) + 8; }
+inline size_t lm_lds_bytes(int rank, int dr) {
+  return 2 * ((size_t)LM_ROWS * lm_ld(rank, dr) + (size_t)LM_KB * lm_ld(rank, dr) + 4 * 16 * LM_PLD) + sizeof(int) * LM_KB;
+}
+
+template <typename T, int NRT>
+__global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const LatentAttnParams p) {
+  extern __shared__ __attribute__((aligned(16))) char sm_raw[];
+  using frag = typename Mfma<T>::frag;
+  using frag4 = typename Mfma16<T>::frag;
+  const int rank = p.rank, dr = p.dr, R = rank + dr;
+  const int RP = (R + 31) & ~31, LD = RP + 8;
+  T* Qs = reinterpret_cast<T*>(sm_raw);                 // [64][LD]
+  T* Ks = Qs + (size_t)LM_ROWS * LD;                    // [32][LD]
+  T* Ps = Ks + (size_t)LM_KB * LD;                      // [4][16][LM_PLD]
+  int* kslot = reinterpret_cast<int*>(Ps + 4 * 16 * LM_PLD);
+  int t0, n;
+  if (p.blocks) {
+    t0 = p.blocks[2 * blockIdx.x];
+    n = p.blocks[2 * blockIdx.x + 1];
+  } else {
+    t0 = blockIdx.x;
+    n = 1;
+  }
+  const int h0 = blockIdx.y * p.hg;
+  const int nh = min(p.hg, p.H - h0);
+  const int M = n * nh;
+  const int split = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, lg = lane >> 4;
+  const T* qa = static_cast<const T*>(p.qa);
+  const T* qr = static_cast<const T*>(p.qr);
+  const T* cache = static_cast<const T*>(p.cache);
+  const int b = p.tok_req ? p.tok_req[t0] : t0;
+  const int64_t p0 = p.positions[t0];
+  const int32_t* table = p.req_to_token + p.req_pool_indices[b] * p.rtt_stride;
+
+  // ---- the keys of this workgroup
+  int64_t j_hi = p0 + n - 1;
+  int64_t j_lo = max((int64_t)0, p0 - (int64_t)p.window + 1);
+  if (p.nsplit > 1) {
+    const int64_t keys = j_hi - j_lo + 1;
+    const int64_t chunk = ((keys + p.nsplit - 1) / p.nsplit + LM_KB - 1) / LM_KB * LM_KB;
+    j_lo += split * chunk;
+    j_hi = min(j_hi, j_lo + chunk - 1);
+  }
+
+  // ---- queries into LDS: absorbed part as is, rope part rotated in fp32 and rounded, padding zero
+  for (int idx = tid; idx < LM_ROWS * RP; idx += 256) {
+    const int m = idx / RP, r = idx - m * RP;
+    float v = 0.f;
+    if (m < M && r < R) {
+      const int ti = m / nh, hi = m - ti * nh;
+      if (r < rank) {
+        v = to_f32(qa[(int64_t)(t0 + ti) * p.qa_st + (int64_t)(h0 + hi) * p.qa_sh + r]);
+      } else {
+        const int i = r - rank, half = p.rot_dims >> 1;
+        const T* src = qr + (int64_t)(t0 + ti) * p.qr_st + (int64_t)(h0 + hi) * p.qr_sh;
+        if (i >= p.rot_dims) {
+          v = to_f32(src[i]);
+        } else {
+          const int f = i < half ? i : i - half;
+          float sn, cs;
+          sincosf((float)(p0 + ti) * p.inv_freq[f], &sn, &cs);
+          const float u = to_f32(src[f]), w = to_f32(src[f + half]);
+          v = i < half ? u * cs - w * sn : w * cs + u * sn;
+        }
+      }
+    }
+    Qs[(size_t)m * LD + r] = from_f32<T>(v);
+  }
+
+  // ---- running softmax state of this lane's four rows (rows 16 wave + 4 lg + r), replicated over the 16 lanes
+  const int r0 = 16 * wave;
+  const bool wave_has_rows = r0 < M;
+  float mrun[4], lrun[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = r0 + 4 * lg + r;
+    const bool with_sink = split == 0 && m < M;
+    mrun[r] = with_sink ? p.sink[h0 + (m % nh)] : -1e30f;
+    lrun[r] = with_sink ? 1.0f : 0.0f;
+  }
+  f32x4 acc[NRT];
+#pragma unroll
+  for (int c = 0; c < NRT; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bool vec_ok = (R % 8 == 0) && aligned16(cache);
+  const int chunks = RP / 8;
+  __syncthreads();
+
+  for (int64_t j0 = j_lo; j0 <= j_hi; j0 += LM_KB) {
+    const int kn = (int)min((int64_t)LM_KB, j_hi - j0 + 1);
+    if (tid < LM_KB) kslot[tid] = tid < kn ? table[j0 + tid] : 0;
+    __syncthreads();
+    for (int idx = tid; idx < LM_KB * chunks; idx += 256) {
+      const int jj = idx / chunks, ch = idx - jj * chunks;
+      Vec<T, 8> v;
+      if (jj < kn && vec_ok && 8 * ch + 8 <= R) {
+        v = ldvec<T, 8>(cache + (int64_t)kslot[jj] * R + 8 * ch);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int r = 8 * ch + e;
+          v.v[e] = (jj < kn && r < R) ? cache[(int64_t)kslot[jj] * R + r] : from_f32<T>(0.f);
+        }
+      }
+      stvec<T, 8>(Ks + (size_t)jj * LD + 8 * ch, v);
+    }
+    __syncthreads();
+    if (wave_has_rows) {
+      // ---- scores of 16 rows x 32 keys
+      f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
+      const T* qrow = Qs + (size_t)(r0 + li) * LD + 8 * lg;
+      const T* k0row = Ks + (size_t)li * LD + 8 * lg;
+      const T* k1row = Ks + (size_t)(16 + li) * LD + 8 * lg;
+      for (int kc = 0; kc < RP; kc += 32) {
+        const frag a = *reinterpret_cast<const frag*>(qrow + kc);
+        s0 = Mfma<T>::run(a, *reinterpret_cast<const frag*>(k0row + kc), s0);
+        s1 = Mfma<T>::run(a, *reinterpret_cast<const frag*>(k1row + kc), s1);
+      }
+      float pr[2][4], alpha[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = r0 + 4 * lg + r;
+        const int64_t pq = p0 + m / nh;
+        float sv[2] = {s0[r], s1[r]};
+        float mx = -INFINITY;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int64_t j = j0 + 16 * h + li;
+          const bool vis = m < M && j <= j_hi && j <= pq && pq - j < p.window;
+          sv[h] = vis ? sv[h] * p.scale : -INFINITY;
+          mx = fmaxf(mx, sv[h]);
+        }
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const float mnew = fmaxf(mrun[r], mx);
+        alpha[r] = expf(mrun[r] - mnew);
+        float sum = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          pr[h][r] = expf(sv[h] - mnew);
+          sum += pr[h][r];
+        }
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o, 64);
+        lrun[r] = lrun[r] * alpha[r] + sum;
+        mrun[r] = mnew;
+      }
+      T* pw = Ps + (size_t)wave * 16 * LM_PLD;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pw[(4 * lg + r) * LM_PLD + li] = from_f32<T>(pr[0][r]);
+        pw[(4 * lg + r) * LM_PLD + 16 + li] = from_f32<T>(pr[1][r]);
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int c = 0; c < NRT; ++c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[c][r] *= alpha[r];
+      // ---- O += P V: two 16-key steps; V = the first `rank` columns of the K tile, read transposed
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const frag4 pa = *reinterpret_cast<const frag4*>(pw + li * LM_PLD + 16 * h + 4 * lg);
+        const T* vrow = Ks + (size_t)(16 * h + 4 * lg + (li >> 2)) * LD + 4 * (li & 3);
+#pragma unroll
+        for (int c = 0; c < NRT; ++c) {
+          if (16 * c < rank) {
+            const auto vb = TrRead<T>::run(vrow + 16 * c);
+            acc[c] = Mfma16<T>::run(pa, __builtin_bit_cast(frag4, vb), acc[c]);
+          }
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+  }
+  if (!wave_has_rows) return;
+  // ---- epilogue: this lane holds rows 16 wave + 4 lg + r, columns 16 c + li
+  T* out = static_cast<T*>(p.out);
+  const T* gate = static_cast<const T*>(p.gate);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int m = r0 + 4 * lg + r;
+    if (m >= M) continue;
+    const int ti = m / nh, hi = m - ti * nh;
+    const int64_t t = t0 + ti;
+    const int h = h0 + hi;
+    if (p.nsplit > 1) {
+      const int64_t cell = ((int64_t)split * p.tokens + t) * p.H + h;
+      if (li == 0) {
+        p.part_m[cell] = mrun[r];
+        p.part_l[cell] = lrun[r];
+      }
+#pragma unroll
+      for (int c = 0; c < NRT; ++c)
+        if (16 * c + li < rank) p.part_o[cell * rank + 16 * c + li] = acc[c][r];
+    } else {
+      float f = 1.0f / lrun[r];
+      if (gate) f *= 1.0f / (1.0f + expf(-to_f32(gate[t * p.gate_st + h])));
+#pragma unroll
+      for (int c = 0; c < NRT; ++c)
+        if (16 * c + li < rank) out[t * p.o_st + (int64_t)h * p.o_sh + 16 * c + li] = from_f32<T>(acc[c][r] * f);
+    }
+  }
+}
+
+// One wave per (token, head): out = sum_i o_i exp(m_i - m) / sum_i l_i exp(m_i - m), times the gate.
+template <typename T>
+__global__ __launch_bounds__(64) void latent_window_merge_kernel(const LatentAttnParams p) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y;
+  float mx = -1e30f;
+  for (int z = 0; z < p.nsplit; ++z) mx = fmaxf(mx, p.part_m[((int64_t)z * p.tokens + t) * p.H + h]);
+  float den = 0.f;
+  for (int z = 0; z < p.nsplit; ++z) {
+    const int64_t cell = ((int64_t)z * p.tokens + t) * p.H + h;
+    den += p.part_l[cell] * expf(p.part_m[cell] - mx);
+  }
+  float f = 1.0f / den;
+  const T* gate = static_cast<const T*>(p.gate);
+  if (gate) f *= 1.0f / (1.0f + expf(-to_f32(gate[t * p.gate_st + h])));
+  T* out = static_cast<T*>(p.out);
+  for (int c = threadIdx.x; c < p.rank; c += 64) {
+    float o = 0.f;
+    for (int z = 0; z < p.nsplit; ++z) {
+      const int64_t cell = ((int64_t)z * p.tokens + t) * p.H + h;
+      o += p.part_o[cell * p.rank + c] * expf(p.part_m[cell] - mx);
+    }
+    out[t * p.o_st + (int64_t)h * p.o_sh + c] = from_f32<T>(o * f);
+  }
+}
+
+template <typename T> inline bool launch_latent_mfma(const LatentAttnParams& p, dim3 grid, size_t lds, hipStream_t st) {
+#define MI355_LM_CASE(N)                                                                                         \
+  {                                                                                                              \
+    auto kern = latent_window_attention_mfma_kernel<T, N>;                                                       \
+    if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, p);                                                       \
+  }
+  const int tiles = (p.rank + 15) / 16;
+  if (tiles <= 4) MI355_LM_CASE(4)
+  else if (tiles <= 8) MI355_LM_CASE(8)
+  else if (tiles <= 16) MI355_LM_CASE(16)
+  else if (tiles <= 32) MI355_LM_CASE(32)
+  else return false;
+#undef MI355_LM_CASE
+  return true;
+}
+
+inline bool latent_mfma_serves(int dtype, int rank, int dr) {
+  return (dtype == MI355_BF16 || dtype == MI355_F16) && rank <= 512 && lm_lds_bytes(rank, dr) <= 160 * 1024;
+}
+
 }  // namespace
 }  // namespace mi355
 
@@ -255,8 +527,9 @@ int mi355_latent_norms_rope_write(void* cq, void* cache, const void* a, const vo
   return MI355_OK;
 }
 
-int mi355_latent_window_attention_block_tokens(int heads, int rank, int rope_dim) {
+int mi355_latent_window_attention_block_tokens(int heads, int rank, int rope_dim, int dtype) {
   if (heads <= 0 || rank <= 0 || rope_dim < 0) return 0;
+  if (latent_mfma_serves(dtype, rank, rope_dim)) return heads >= LM_ROWS ? 1 : LM_ROWS / heads;
   const LatentAttnPlan pl = plan_latent_attn(heads, rank, rope_dim);
   return pl.lds <= 160 * 1024 ? pl.bq : 0;
 }
@@ -267,7 +540,7 @@ int mi355_latent_window_attention(void* out, const void* qa, const void* qr, con
                                   const float* inv_freq, int64_t qa_token_stride, int64_t qa_head_stride, int64_t qr_token_stride,
                                   int64_t qr_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t gate_stride,
                                   int64_t req_to_token_stride, int heads, int rank, int rope_dim, int rot_dims, int window,
-                                  float scale, int dtype, void* stream) {
+                                  float scale, int num_splits, float* split_scratch, int64_t tokens, int dtype, void* stream) {
   MI355_REQUIRE(out && qa && cache && req_to_token && req_pool_indices && positions && sink, MI355_ERR_INVALID,
                 "latent_window_attention: null pointer");
   MI355_REQUIRE(rope_dim == 0 || (qr && inv_freq), MI355_ERR_INVALID, "latent_window_attention: the rope part needs qr and inv_freq");
@@ -275,7 +548,16 @@ int mi355_latent_window_attention(void* out, const void* qa, const void* qr, con
                     num_blocks >= 0 && num_blocks < (1ll << 31),
                 MI355_ERR_INVALID, "latent_window_attention: bad shape");
   if (num_blocks == 0) return MI355_OK;
-  const LatentAttnPlan pl = plan_latent_attn(heads, rank, rope_dim);
+  const bool mfma = latent_mfma_serves(dtype, rank, rope_dim);
+  MI355_REQUIRE(num_splits >= 1 && num_splits <= 64 && (num_splits == 1 || (mfma && blocks == nullptr && split_scratch && tokens == num_blocks)),
+                MI355_ERR_INVALID, "latent_window_attention: key splits need the 16-bit kernel, one token per run and a scratch array");
+  LatentAttnPlan pl = plan_latent_attn(heads, rank, rope_dim);
+  if (mfma) {
+    pl.hg = std::min(heads, LM_ROWS);
+    pl.bq = heads >= LM_ROWS ? 1 : LM_ROWS / heads;
+    pl.kb = LM_KB;
+    pl.lds = lm_lds_bytes(rank, rope_dim);
+  }
   MI355_REQUIRE(pl.lds <= 160 * 1024, MI355_ERR_UNSUPPORTED, "latent_window_attention: rank %d + rope %d does not fit the LDS tile", rank,
                 rope_dim);
   LatentAttnParams p;
@@ -286,6 +568,25 @@ int mi355_latent_window_attention(void* out, const void* qa, const void* qr, con
   p.o_st = out_token_stride; p.o_sh = out_head_stride; p.gate_st = gate_stride; p.rtt_stride = req_to_token_stride;
   p.H = heads; p.rank = rank; p.dr = rope_dim; p.rot_dims = rot_dims; p.window = window; p.hg = pl.hg; p.kb = pl.kb; p.rows_cap = pl.hg * pl.bq;
   p.scale = scale;
+  p.nsplit = num_splits; p.tokens = tokens;
+  p.part_o = split_scratch;
+  p.part_m = split_scratch ? split_scratch + (int64_t)num_splits * tokens * heads * rank : nullptr;
+  p.part_l = split_scratch ? p.part_m + (int64_t)num_splits * tokens * heads : nullptr;
+  if (mfma) {
+    const dim3 mgrid((unsigned)num_blocks, (unsigned)((heads + pl.hg - 1) / pl.hg), (unsigned)num_splits);
+    bool ok = false;
+    if (dtype == MI355_BF16) ok = launch_latent_mfma<bf16_t>(p, mgrid, pl.lds, (hipStream_t)stream);
+    else ok = launch_latent_mfma<f16_t>(p, mgrid, pl.lds, (hipStream_t)stream);
+    MI355_REQUIRE(ok, MI355_ERR_UNSUPPORTED, "latent_window_attention: rank %d is not served", rank);
+    MI355_CHECK_LAUNCH("latent_window_attention");
+    if (num_splits > 1) {
+      const dim3 g2((unsigned)tokens, (unsigned)heads);
+      if (dtype == MI355_BF16) hipLaunchKernelGGL((latent_window_merge_kernel<bf16_t>), g2, dim3(64), 0, (hipStream_t)stream, p);
+      else hipLaunchKernelGGL((latent_window_merge_kernel<f16_t>), g2, dim3(64), 0, (hipStream_t)stream, p);
+      MI355_CHECK_LAUNCH("latent_window_attention (merge)");
+    }
+    return MI355_OK;
+  }
   const dim3 grid((unsigned)num_blocks, (unsigned)((heads + pl.hg - 1) / pl.hg), 1);
   MI355_DISPATCH_DTYPE(dtype, "latent_window_attention", {
     auto kern = latent_window_attention_kernel<T>;

@@ -297,14 +297,19 @@ class Mi355AttnBackend(AttentionBackend):
         The new tokens' rows are in the cache already (ops.latent_norms_rope_write); prefill portions, decode steps and
         mixed batches are the same launch, told apart only by the list of token runs."""
         ops = get_ops()
-        bq = ops.latent_window_attention_block_tokens(layer.tp_q_head_num, layer.kv_rank, layer.rope_dim)
+        bq = ops.latent_window_attention_block_tokens(layer.tp_q_head_num, layer.kv_rank, layer.rope_dim, qa.dtype)
         if bq <= 0:
             raise NotImplementedError(f"latent window attention: rank {layer.kv_rank} + rope {layer.rope_dim} is not served")
         cache = forward_batch.token_to_kv_pool.get_key_buffer(layer.layer_id)
+        splits = 1
+        if forward_batch.forward_mode.is_decode() and forward_batch.seq_lens_cpu is not None:
+            # a decode step has few workgroups: long windows are cut into key ranges that a second launch merges
+            splits = ops.latent_window_attention_splits(qa.shape[0], layer.tp_q_head_num, layer.kv_rank, layer.window,
+                                                        int(forward_batch.seq_lens_cpu.max()) - 1, qa.dtype)
         return ops.latent_window_attention(
             qa, qr, cache, out, forward_batch.req_to_token_pool.req_to_token, forward_batch.req_pool_indices,
             forward_batch.positions, layer.sink.data, layer.inv_freq, layer.rot_dims, layer.window, layer.scaling, gate=gate,
-            tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq))
+            tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq), num_splits=splits)
 
     def _windowed(self, layer) -> bool:
         """triton_backend.py:656, 711: a layer with sliding_window_size > -1 attends the window lists."""

@@ -1207,15 +1207,25 @@ def latent_norms_rope_write(a: torch.Tensor, q_weight: torch.Tensor, kv_weight: 
     return cq
 
 
-def latent_window_attention_block_tokens(heads: int, rank: int, rope_dim: int) -> int:
+def latent_window_attention_block_tokens(heads: int, rank: int, rope_dim: int, dtype: torch.dtype) -> int:
     """Most consecutive tokens of one sequence that a workgroup of latent_window_attention takes (0: shape not served)."""
-    return int(_lib_().mi355_latent_window_attention_block_tokens(heads, rank, rope_dim))
+    return int(_lib_().mi355_latent_window_attention_block_tokens(heads, rank, rope_dim, _DT[dtype]))
+
+
+def latent_window_attention_splits(tokens: int, heads: int, rank: int, window: int, max_position: int, dtype: torch.dtype) -> int:
+    """Key ranges per token for a decode-sized launch of the 16-bit kernel: enough workgroups to cover the chip twice,
+    at least 128 keys each."""
+    if dtype not in (torch.bfloat16, torch.float16) or rank > 512:
+        return 1
+    keys = min(window, max_position + 1)
+    wgs = max(1, tokens * ((heads + 63) // 64))
+    return int(max(1, min(64, (512 + wgs - 1) // wgs, keys // 128)))
 
 
 def latent_window_attention(qa: torch.Tensor, qr: torch.Tensor, cache: torch.Tensor, out: torch.Tensor, req_to_token: torch.Tensor,
                             req_pool_indices: torch.Tensor, positions: torch.Tensor, sink: torch.Tensor, inv_freq: torch.Tensor,
                             rot_dims: int, window: int, scale: float, gate: Optional[torch.Tensor] = None, tok_req=None,
-                            blocks=None) -> torch.Tensor:
+                            blocks=None, num_splits: int = 1) -> torch.Tensor:
     """qa [T, H, rank] and out [T, H, rank] (any token / head strides), qr [T, H, rope_dim] unrotated, cache
     [slots, rank + rope_dim], gate [T, H] logits (row-strided) or None, blocks int32 [n, 2] runs of tokens or None."""
     _gpu(qa, qr, cache, out, req_to_token, req_pool_indices, positions, sink, inv_freq, gate, tok_req, blocks)
@@ -1233,10 +1243,14 @@ def latent_window_attention(qa: torch.Tensor, qr: torch.Tensor, cache: torch.Ten
         nb = blocks.shape[0]
     else:
         nb = T
+    scratch = None
+    if num_splits > 1:
+        assert blocks is None, "key splits serve launches of one token per run"
+        scratch = torch.empty(num_splits * T * H * (rank + 2), dtype=torch.float32, device=qa.device)
     check(_lib_().mi355_latent_window_attention(
         out.data_ptr(), qa.data_ptr(), _p(qr) if rope_dim else None, cache.data_ptr(), _p(gate), req_to_token.data_ptr(),
         req_pool_indices.data_ptr(), _p(tok_req), positions.data_ptr(), _p(blocks), nb, sink.data_ptr(), _p(inv_freq),
         qa.stride(0), qa.stride(1), qr.stride(0) if rope_dim else 0, qr.stride(1) if rope_dim else 0, out.stride(0), out.stride(1),
         gate.stride(0) if gate is not None else 0, req_to_token.stride(0), H, rank, rope_dim, rot_dims, int(window), float(scale),
-        _dt(qa), _stream(qa)), "latent_window_attention")
+        int(num_splits), _p(scratch), T, _dt(qa), _stream(qa)), "latent_window_attention")
     return out

@@ -289,12 +289,16 @@ def latent_norms_rope_write(a, q_weight, kv_weight, positions, out_cache_loc, in
     return cq
 
 
-def latent_window_attention_block_tokens(heads, rank, rope_dim):
+def latent_window_attention_block_tokens(heads, rank, rope_dim, dtype):
     return 3
 
 
+def latent_window_attention_splits(tokens, heads, rank, window, max_position, dtype):
+    return 1
+
+
 def latent_window_attention(qa, qr, cache, out, req_to_token, req_pool_indices, positions, sink, inv_freq, rot_dims, window,
-                            scale, gate=None, tok_req=None, blocks=None):
+                            scale, gate=None, tok_req=None, blocks=None, num_splits=1):
     T, H, rank = qa.shape
     covered = torch.zeros(T, dtype=torch.bool)
     runs = [(t, 1) for t in range(T)] if blocks is None else [(int(a), int(n)) for a, n in blocks.tolist()]

@@ -160,7 +160,7 @@ def test_latent_norms_rope_write_and_attention(dtype, tol, H, rank, dr, rot_dims
     req_to_token = torch.zeros(3, n + 5, dtype=torch.int32)
     req_to_token[1, :n] = slots.to(torch.int32)
     common = dict(req_to_token=req_to_token.to(DEV), sink=sink.to(DEV), inv_freq=inv_freq, rot_dims=rot_dims, window=window, scale=scale)
-    bq = ops().latent_window_attention_block_tokens(H, rank, dr)
+    bq = ops().latent_window_attention_block_tokens(H, rank, dr, dtype)
     assert bq >= 1
 
     def blocks_of(portions):
@@ -170,7 +170,7 @@ def test_latent_norms_rope_write_and_attention(dtype, tol, H, rank, dr, rot_dims
             t0 += m
         return torch.tensor(out, dtype=torch.int32, device=DEV)
 
-    def run(lo, portions, as_decode=False):
+    def run(lo, portions, as_decode=False, num_splits=1):
         """Tokens lo .. of the sequence as one extend batch whose requests are the given portions of it (each request
         the same sequence, with its own prefix), or as a decode batch."""
         m = sum(portions)
@@ -180,13 +180,18 @@ def test_latent_norms_rope_write_and_attention(dtype, tol, H, rank, dr, rot_dims
                                                                  torch.tensor(portions)).to(DEV)
         ops().latent_window_attention(
             qa[idx].to(DEV), qr[idx].to(DEV), cache, out.transpose(0, 1), req_pool_indices=torch.ones(m if as_decode else len(portions), dtype=torch.int64, device=DEV),
-            positions=pos[idx].to(DEV), gate=gate[idx].to(DEV), tok_req=tok_req, blocks=None if as_decode else blocks_of(portions), **common)
+            positions=pos[idx].to(DEV), gate=gate[idx].to(DEV), tok_req=tok_req, blocks=None if as_decode else blocks_of(portions),
+            num_splits=num_splits, **common)
         return out.transpose(0, 1).cpu().double()
 
     lim = tol * 4 * max(1.0, float(want.abs().max()))
     assert (run(0, [n]) - want).abs().max() < lim
     assert (run(0, [2, 11, 1, 17, n - 31]) - want).abs().max() < lim
     assert (run(n - 9, [1] * 9, as_decode=True) - want[n - 9:]).abs().max() < lim
+    if dtype != torch.float32 and rank <= 512:
+        # the keys of every token cut into ranges (some of them empty, one holding the sink) and merged
+        for splits in (2, 3, 7):
+            assert (run(n - 9, [1] * 9, as_decode=True, num_splits=splits) - want[n - 9:]).abs().max() < lim
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -214,11 +219,11 @@ def test_window_edges_far_keys_and_the_sink_show(dtype):
             rows[planted, 0] = 8.0
             qa[:, :, 0] = 8.0
         if planted is not None and plant_in_rope:
-            # the same through the rope part: key and query rotate by their own positions, so the planted key is
-            # written as the rotation of the query's direction by (p - planted) steps back
+            # the same through the rope part: the cache holds rotated keys and the kernel rotates the query by its own
+            # position p, so the planted row is the query's direction turned by p
             k = torch.zeros(1, 1, dr, dtype=torch.float64)
             k[..., 0] = 8.0
-            rows[planted, rank:] = ref.rotate_half(k, torch.tensor([planted]), 10000.0, dr)[0, 0].to(dtype)
+            rows[planted, rank:] = ref.rotate_half(k, torch.tensor([p]), 10000.0, dr)[0, 0].to(dtype)
             qr[..., 0] = 8.0
         cache[req_to_token[0].long()] = rows.to(DEV)
         out = torch.zeros(1, H, rank, dtype=dtype, device=DEV)
