@@ -1,0 +1,227 @@
+"""Side-by-side throughput of two model designs at equal layer sizes (random weights, synthetic prompts): prefill
+tokens/s of a batch of whole prompts, decode tokens/s of a static batch, and each design's hot kernels alone with the
+bytes or flops their algorithm moves against the HBM3E / matrix-core peaks.  Started by `bench.py --design-compare`;
+the default workload of bench.py does not pass through here.
+
+Seturax is compared with the package's closest model, the dense DeepSeek stack (multi-head latent attention): same
+width, heads, head widths, latent ranks, feed-forward width, depth and vocabulary; Seturax's window is a parameter of
+the size."""
+import time
+
+import torch
+
+HBM_PEAK = 8.0e12
+MFMA_BF16_PEAK = 2.5e15
+
+SIZES = {
+    # DeepSeek-like attention geometry (16 / 32 heads of 128 + 64, latent 512, q latent 1536) on two widths
+    "w2048": dict(width=2048, heads=16, nope=128, rope=64, v=128, kv_rank=512, q_rank=1536, ff=8192, layers=4, vocab=32768, window=1024),
+    "w4096": dict(width=4096, heads=32, nope=128, rope=64, v=128, kv_rank=512, q_rank=1536, ff=12288, layers=4, vocab=32768, window=1024),
+    "tiny": dict(width=256, heads=16, nope=128, rope=64, v=128, kv_rank=512, q_rank=192, ff=512, layers=2, vocab=2048, window=128),
+}
+
+
+def seturax_config(s: dict) -> dict:
+    mixer = dict(heads=s["heads"], dim=s["nope"], rot_dim=s["rope"], vdim=s["v"], kv_rank=s["kv_rank"], q_rank=s["q_rank"],
+                 mask=dict(size=s["window"]), rot=dict(base=10000.0, dims=s["rope"]), scale=(s["nope"] + s["rope"]) ** -0.5)
+    return dict(architecture="Seturax", vocab=s["vocab"], width=s["width"], logit_scale=1.0, norm=dict(eps=1e-6),
+                embedding=dict(scale=1.0, bigram=dict(buckets=65521, mul_prev=8191, mul_cur=127)),
+                layers=[dict(type="latent_attention", mixer=mixer, mlp=dict(kind="dense", ff=s["ff"])) for _ in range(s["layers"])])
+
+
+def deepseek_config(s: dict, dtype: str) -> dict:
+    return dict(architectures=["DeepseekV3ForCausalLM"], model_type="deepseek_v3", hidden_size=s["width"],
+                num_hidden_layers=s["layers"], num_attention_heads=s["heads"], q_lora_rank=s["q_rank"], kv_lora_rank=s["kv_rank"],
+                qk_nope_head_dim=s["nope"], qk_rope_head_dim=s["rope"], v_head_dim=s["v"], intermediate_size=s["ff"],
+                vocab_size=s["vocab"], rms_norm_eps=1e-6, rope_theta=10000.0, max_position_embeddings=16384, rope_scaling=None,
+                n_routed_experts=None, first_k_dense_replace=s["layers"], tie_word_embeddings=False, torch_dtype=dtype)
+
+
+def _timed(fn, reps: int, warmup: int = 2) -> float:
+    """Seconds per call, device time between two events."""
+    for _ in range(warmup):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / reps
+
+
+def _runner(cfg: dict, dtype: str, tokens: int, reqs: int, ctx: int, graph: bool):
+    from .configs.model_config import ModelConfig
+    from .model_executor.model_runner import ModelRunner
+    from .server_args import ServerArgs
+
+    sa = ServerArgs(dtype=dtype, max_total_tokens=tokens, max_running_requests=reqs, context_length=ctx,
+                    disable_cuda_graph=not graph, cuda_graph_bs=[reqs - 8] if graph else None, graph_capture_fallback=True)
+    return ModelRunner(ModelConfig(cfg, dtype=dtype, context_length=ctx), sa)
+
+
+def model_throughput(cfg: dict, dtype: str, prefill_bs: int, prefill_len: int, decode_bs: int, decode_ctx: int, steps: int,
+                     graph: bool) -> dict:
+    from . import bench_one_batch as bob
+
+    ctx = max(prefill_len, decode_ctx + steps + 8) + 16
+    mr = _runner(cfg, dtype, max(prefill_bs * prefill_len, decode_bs * (decode_ctx + steps + 8)) + 64, max(prefill_bs, decode_bs) + 8,
+                 ctx, graph)
+    vocab = mr.model_config.vocab_size
+
+    def fresh(bs, n):
+        bob.clear_pools(mr)
+        return bob.prepare_synthetic_inputs_for_latency_test(bs, n, seed=0, vocab=vocab)
+
+    times = []
+    for r in range(3):
+        reqs = fresh(prefill_bs, prefill_len)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        bob.extend(reqs, mr)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    prefill_s = min(times[1:])
+    reqs = fresh(decode_bs, decode_ctx)
+    nxt, _, batch = bob.extend(reqs, mr)
+    for _ in range(4):
+        nxt, _ = bob.decode(nxt, batch, mr)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        nxt, _ = bob.decode(nxt, batch, mr)
+    torch.cuda.synchronize()
+    decode_s = (time.perf_counter() - t0) / steps
+    out = dict(prefill_tok_s=round(prefill_bs * prefill_len / prefill_s), prefill_ms=round(prefill_s * 1e3, 2),
+               decode_tok_s=round(decode_bs / decode_s), decode_ms_per_step=round(decode_s * 1e3, 3),
+               graph=mr.graph_runner is not None)
+    del mr
+    torch.cuda.empty_cache()
+    return out
+
+
+def attention_kernels(s: dict, bs: int, ctx: int, prefill_bs: int, prefill_len: int) -> dict:
+    """The two designs' attention launches alone, bf16.  Decode: bytes = every visible cache row once per sequence.
+    Prefill: flops of the form each kernel computes (absorbed: 2 (2 rank + rope) per query-key pair and head;
+    expanded multi-head: 2 (nope + rope + v))."""
+    from . import ops
+    from .layers.rotary_embedding import rotate_half_inv_freq
+
+    dev, dt = "cuda", torch.bfloat16
+    H, rank, rope, W = s["heads"], s["kv_rank"], s["rope"], s["window"]
+    R = rank + rope
+    g = torch.Generator(device=dev).manual_seed(0)
+    slots = bs * ctx + 8
+    cache = torch.randn(slots, R, device=dev, generator=g).to(dt)
+    req_to_token = (torch.arange(bs * ctx, device=dev, dtype=torch.int32) + 1).view(bs, ctx)
+    rpi = torch.arange(bs, device=dev)
+    qa = torch.randn(bs, H, rank, device=dev, generator=g).to(dt)
+    qr = torch.randn(bs, H, rope, device=dev, generator=g).to(dt)
+    out = torch.empty_like(qa)
+    sink = torch.zeros(H, device=dev)
+    inv_freq = rotate_half_inv_freq(10000.0, rope).to(dev)
+    pos = torch.full((bs,), ctx - 1, device=dev, dtype=torch.int64)
+    res = {}
+    keys = min(W, ctx)
+    splits = ops.latent_window_attention_splits(bs, H, rank, W, ctx - 1, dt)
+    t = _timed(lambda: ops.latent_window_attention(qa, qr, cache, out, req_to_token, rpi, pos, sink, inv_freq, rope, W, 0.07,
+                                                   num_splits=splits), 20)
+    b = bs * keys * R * 2
+    res["seturax_decode_attention"] = dict(us=round(t * 1e6, 1), keys=keys, splits=splits, gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
+    # the closest model's decode attention over the same rows (no window: all ctx rows)
+    q = torch.cat([qa, qr], -1).contiguous()
+    o2 = torch.empty(bs, H, rank, device=dev, dtype=dt)
+    seq = torch.full((bs,), keys, device=dev, dtype=torch.int64)
+    nsp = max(1, min(64, (512 + bs * ((H + 15) // 16) - 1) // (bs * ((H + 15) // 16)), keys // 256))
+    logits = torch.empty(bs * H * nsp * rank, device=dev, dtype=torch.float32)
+    lse = torch.empty(bs * H * nsp, device=dev, dtype=torch.float32)
+    tickets = torch.zeros(max(bs * H, 1024), device=dev, dtype=torch.int32)
+    chunk = torch.full((1,), (keys + nsp - 1) // nsp, device=dev, dtype=torch.int32)
+    t = _timed(lambda: ops.decode_attention_mla(q, cache.view(slots, 1, R), o2, req_to_token, rpi, seq, logits if nsp > 1 else None,
+                                                lse if nsp > 1 else None, nsp, rank, 0.07, 0.0, tickets=tickets if nsp > 1 else None,
+                                                kv_chunk_keys=chunk if nsp > 1 else None), 20)
+    b = bs * keys * R * 2
+    res["deepseek_decode_attention"] = dict(us=round(t * 1e6, 1), keys=keys, splits=nsp, gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
+    # prefill: whole prompts, every token a query
+    T = prefill_bs * prefill_len
+    cache_p = torch.randn(T + 8, R, device=dev, generator=g).to(dt)
+    rtt = (torch.arange(T, device=dev, dtype=torch.int32) + 1).view(prefill_bs, prefill_len)
+    qa = torch.randn(T, H, rank, device=dev, generator=g).to(dt)
+    qr = torch.randn(T, H, rope, device=dev, generator=g).to(dt)
+    out = torch.empty_like(qa)
+    posp = torch.arange(prefill_len, device=dev).repeat(prefill_bs)
+    tok_req = torch.repeat_interleave(torch.arange(prefill_bs, device=dev, dtype=torch.int32), prefill_len)
+    bq = ops.latent_window_attention_block_tokens(H, rank, rope, dt)
+    starts = torch.arange(0, T, bq, dtype=torch.int32)
+    blocks = torch.stack([starts, torch.full_like(starts, bq)], 1).to(dev)     # prefill_len is a multiple of bq here
+    assert prefill_len % bq == 0
+    t = _timed(lambda: ops.latent_window_attention(qa, qr, cache_p, out, rtt, torch.arange(prefill_bs, device=dev), posp, sink, inv_freq,
+                                                   rope, W, 0.07, tok_req=tok_req, blocks=blocks), 5)
+    pairs = prefill_bs * sum(min(p + 1, W) for p in range(prefill_len))
+    fl = pairs * H * 2 * (2 * rank + rope)
+    res["seturax_prefill_attention"] = dict(ms=round(t * 1e3, 3), tflops=round(fl / t / 1e12, 1), of_mfma_peak=round(fl / t / MFMA_BF16_PEAK, 3),
+                                            form="absorbed, window %d" % W)
+    # the closest model's prefill: expanded multi-head attention, causal, no window
+    nope, vd = s["nope"], s["v"]
+    qm = torch.randn(T, H, nope + rope, device=dev, generator=g).to(dt)
+    km = torch.randn(T, H, nope + rope, device=dev, generator=g).to(dt)
+    vm = torch.randn(T, H, vd, device=dev, generator=g).to(dt)
+    om = torch.empty(T, H, vd, device=dev, dtype=dt)
+    qo = torch.arange(0, T + 1, prefill_len, device=dev, dtype=torch.int32)
+    kvp = torch.zeros(prefill_bs + 1, device=dev, dtype=torch.int32)
+    dummy = torch.zeros(1, device=dev, dtype=torch.int32)
+    t = _timed(lambda: ops.extend_attention_fwd(qm, km, vm, om, km, vm, qo, kvp, dummy, None, True, None, prefill_len, 0.07, 0.0), 5)
+    pairs = prefill_bs * prefill_len * (prefill_len + 1) // 2
+    fl = pairs * H * 2 * (nope + rope + vd)
+    res["deepseek_prefill_attention"] = dict(ms=round(t * 1e3, 3), tflops=round(fl / t / 1e12, 1), of_mfma_peak=round(fl / t / MFMA_BF16_PEAK, 3),
+                                             form="expanded multi-head, causal over %d" % prefill_len)
+    return res
+
+
+def stream_kernels(s: dict, tokens: int) -> dict:
+    """The elementwise launches of a layer beside the closest model's like ones, by bytes moved (bf16 activations)."""
+    from . import ops
+
+    dev, dt = "cuda", torch.bfloat16
+    D, ff = s["width"], s["ff"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(tokens, D, device=dev, generator=g)
+    w = torch.ones(D, device=dev, dtype=dt)
+    state = torch.zeros(8, D, device=dev)
+    r2s = torch.ones(tokens, device=dev, dtype=torch.int32)
+    rpi = torch.arange(tokens, device=dev)
+    pos = torch.arange(1, tokens + 1, device=dev)
+    hl = torch.empty(tokens, D, device=dev)
+    res = {}
+    t = _timed(lambda: ops.layernorm_shift(x, w, 1e-6, shift=w, state=state, req_to_state=r2s, req_pool_indices=rpi, positions=pos, h_last=hl), 20)
+    b = tokens * D * (4 + 4 + 2 + 2 + 4)     # x and the state row in, h and hs out, h_last out
+    res["layernorm_shift"] = dict(us=round(t * 1e6, 1), gbs=round(b / t / 1e9))
+    xb, rb = x.to(dt), x.to(dt)
+    t = _timed(lambda: ops.fused_add_rmsnorm(xb, rb, w, 1e-6), 20)
+    res["fused_add_rmsnorm (closest)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * 2 * 4 / t / 1e9))
+    hp = torch.randn(tokens, 2 * ff + 2 * D, device=dev, generator=g).to(dt)
+    t = _timed(lambda: ops.gelu_tanh_and_mul(hp[:, :ff], hp[:, ff: 2 * ff]), 20)
+    res["gelu_tanh_and_mul"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * ff * 2 * 3 / t / 1e9))
+    gu = hp[:, : 2 * ff].contiguous()
+    t = _timed(lambda: ops.silu_and_mul(gu), 20)
+    res["silu_and_mul (closest)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * ff * 2 * 3 / t / 1e9))
+    y1, y2 = x.to(dt), x.to(dt)
+    t = _timed(lambda: ops.gated_residual_add(x, hp[:, 2 * ff: 2 * ff + D], w, y1, hp[:, 2 * ff + D:], w, y2), 20)
+    res["gated_residual_add"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (8 + 8) / t / 1e9))
+    return res
+
+
+def run(size: str, dtype: str = "bfloat16", steps: int = 32, prefill_bs: int = 4, prefill_len: int = 2048, decode_bs: int = 64,
+        decode_ctx: int = 1024) -> dict:
+    from .model_loader.synthetic import hf_config_dict  # noqa: F401  (the package's presets stay as they are)
+
+    s = SIZES[size]
+    out = dict(size=size, shape=s, dtype=dtype, data="synthetic", workload=dict(prefill=[prefill_bs, prefill_len], decode=[decode_bs, decode_ctx], steps=steps))
+    out["seturax"] = model_throughput(seturax_config(s), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=False)
+    out["deepseek_dense"] = model_throughput(deepseek_config(s, dtype), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=True)
+    out["deepseek_dense_eager"] = model_throughput(deepseek_config(s, dtype), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=False)
+    out["attention"] = attention_kernels(s, decode_bs, decode_ctx, prefill_bs, prefill_len)
+    out["stream_kernels_decode"] = stream_kernels(s, decode_bs)
+    out["stream_kernels_prefill"] = stream_kernels(s, prefill_bs * prefill_len)
+    return out

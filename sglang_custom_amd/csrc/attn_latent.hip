@@ -251,11 +251,13 @@ constexpr int LM_ROWS = 64;
 constexpr int LM_PLD = LM_KB + 8;
 
 inline int lm_ld(int rank, int dr) { return ((rank + dr + 31) & ~31) + 8; }
-inline size_t lm_lds_bytes(int rank, int dr) {
-  return 2 * ((size_t)LM_ROWS * lm_ld(rank, dr) + (size_t)LM_KB * lm_ld(rank, dr) + 4 * 16 * LM_PLD) + sizeof(int) * LM_KB;
+inline size_t lm_lds_bytes(int rank, int dr, int rows = LM_ROWS) {
+  return 2 * ((size_t)rows * lm_ld(rank, dr) + (size_t)LM_KB * lm_ld(rank, dr) + 4 * 16 * LM_PLD) + sizeof(int) * LM_KB;
 }
 
-template <typename T, int NRT>
+// ROWS: query rows the workgroup holds (64; 16 for decode steps of models with at most 16 heads, where only the first
+// wave has rows: the smaller Q tile lets two workgroups share a CU while the other waves still help load the K tiles)
+template <typename T, int NRT, int ROWS>
 __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const LatentAttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char sm_raw[];
   using frag = typename Mfma<T>::frag;
@@ -263,7 +265,7 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
   const int rank = p.rank, dr = p.dr, R = rank + dr;
   const int RP = (R + 31) & ~31, LD = RP + 8;
   T* Qs = reinterpret_cast<T*>(sm_raw);                 // [64][LD]
-  T* Ks = Qs + (size_t)LM_ROWS * LD;                    // [32][LD]
+  T* Ks = Qs + (size_t)ROWS * LD;                       // [32][LD]
   T* Ps = Ks + (size_t)LM_KB * LD;                      // [4][16][LM_PLD]
   int* kslot = reinterpret_cast<int*>(Ps + 4 * 16 * LM_PLD);
   int t0, n;
@@ -297,7 +299,7 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
   }
 
   // ---- queries into LDS: absorbed part as is, rope part rotated in fp32 and rounded, padding zero
-  for (int idx = tid; idx < LM_ROWS * RP; idx += 256) {
+  for (int idx = tid; idx < ROWS * RP; idx += 256) {
     const int m = idx / RP, r = idx - m * RP;
     float v = 0.f;
     if (m < M && r < R) {
@@ -323,7 +325,7 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
 
   // ---- running softmax state of this lane's four rows (rows 16 wave + 4 lg + r), replicated over the 16 lanes
   const int r0 = 16 * wave;
-  const bool wave_has_rows = r0 < M;
+  const bool wave_has_rows = r0 < M && r0 < ROWS;
   float mrun[4], lrun[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -364,7 +366,23 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
       const T* qrow = Qs + (size_t)(r0 + li) * LD + 8 * lg;
       const T* k0row = Ks + (size_t)li * LD + 8 * lg;
       const T* k1row = Ks + (size_t)(16 + li) * LD + 8 * lg;
-      for (int kc = 0; kc < RP; kc += 32) {
+      // three 32-wide chunks per round: nine LDS reads in flight before the six products that use them
+      int kc = 0;
+      for (; kc + 96 <= RP; kc += 96) {
+        frag a[3], b0[3], b1[3];
+#pragma unroll
+        for (int u = 0; u < 3; ++u) {
+          a[u] = *reinterpret_cast<const frag*>(qrow + kc + 32 * u);
+          b0[u] = *reinterpret_cast<const frag*>(k0row + kc + 32 * u);
+          b1[u] = *reinterpret_cast<const frag*>(k1row + kc + 32 * u);
+        }
+#pragma unroll
+        for (int u = 0; u < 3; ++u) {
+          s0 = Mfma<T>::run(a[u], b0[u], s0);
+          s1 = Mfma<T>::run(a[u], b1[u], s1);
+        }
+      }
+      for (; kc < RP; kc += 32) {
         const frag a = *reinterpret_cast<const frag*>(qrow + kc);
         s0 = Mfma<T>::run(a, *reinterpret_cast<const frag*>(k0row + kc), s0);
         s1 = Mfma<T>::run(a, *reinterpret_cast<const frag*>(k1row + kc), s1);
@@ -409,16 +427,28 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
       for (int c = 0; c < NRT; ++c)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[c][r] *= alpha[r];
-      // ---- O += P V: two 16-key steps; V = the first `rank` columns of the K tile, read transposed
+      // ---- O += P V on the k = 32 instruction: lane group lg supplies keys 8 lg .. 8 lg + 7 of the tile, as two
+      // transposed reads of four keys each; V = the first `rank` columns of the K tile.  Eight column tiles per
+      // round, all sixteen reads issued before the eight products.
+      const frag pa = *reinterpret_cast<const frag*>(pw + li * LM_PLD + 8 * lg);
+      const T* vrow = Ks + (size_t)(8 * lg + (li >> 2)) * LD + 4 * (li & 3);
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const frag4 pa = *reinterpret_cast<const frag4*>(pw + li * LM_PLD + 16 * h + 4 * lg);
-        const T* vrow = Ks + (size_t)(16 * h + 4 * lg + (li >> 2)) * LD + 4 * (li & 3);
+      for (int c0 = 0; c0 < NRT; c0 += 8) {
+        if (16 * c0 < rank) {
+          typename TrRead<T>::v4 lo[8], hi[8];
 #pragma unroll
-        for (int c = 0; c < NRT; ++c) {
-          if (16 * c < rank) {
-            const auto vb = TrRead<T>::run(vrow + 16 * c);
-            acc[c] = Mfma16<T>::run(pa, __builtin_bit_cast(frag4, vb), acc[c]);
+          for (int u = 0; u < 8; ++u) {
+            if (c0 + u < NRT) {
+              lo[u] = TrRead<T>::run(vrow + 16 * (c0 + u));
+              hi[u] = TrRead<T>::run(vrow + 4 * LD + 16 * (c0 + u));
+            }
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            if (c0 + u < NRT) {
+              typename TrRead<T>::v4 both[2] = {lo[u], hi[u]};
+              acc[c0 + u] = Mfma<T>::run(pa, __builtin_bit_cast(frag, both), acc[c0 + u]);
+            }
           }
         }
       }
@@ -456,38 +486,66 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
   }
 }
 
-// One wave per (token, head): out = sum_i o_i exp(m_i - m) / sum_i l_i exp(m_i - m), times the gate.
+// One workgroup per (token, head): out = sum_i o_i exp(m_i - m) / sum_i l_i exp(m_i - m), times the gate.  The split
+// weights are computed once into LDS; every thread then sums four columns at a time.
 template <typename T>
-__global__ __launch_bounds__(64) void latent_window_merge_kernel(const LatentAttnParams p) {
+__global__ __launch_bounds__(128) void latent_window_merge_kernel(const LatentAttnParams p) {
+  __shared__ float wz[64];
+  __shared__ float fsh;
   const int64_t t = blockIdx.x;
   const int h = blockIdx.y;
-  float mx = -1e30f;
-  for (int z = 0; z < p.nsplit; ++z) mx = fmaxf(mx, p.part_m[((int64_t)z * p.tokens + t) * p.H + h]);
-  float den = 0.f;
-  for (int z = 0; z < p.nsplit; ++z) {
+  const int ns = p.nsplit;
+  if (threadIdx.x < 64) {
+    const int z = threadIdx.x;
     const int64_t cell = ((int64_t)z * p.tokens + t) * p.H + h;
-    den += p.part_l[cell] * expf(p.part_m[cell] - mx);
-  }
-  float f = 1.0f / den;
-  const T* gate = static_cast<const T*>(p.gate);
-  if (gate) f *= 1.0f / (1.0f + expf(-to_f32(gate[t * p.gate_st + h])));
-  T* out = static_cast<T*>(p.out);
-  for (int c = threadIdx.x; c < p.rank; c += 64) {
-    float o = 0.f;
-    for (int z = 0; z < p.nsplit; ++z) {
-      const int64_t cell = ((int64_t)z * p.tokens + t) * p.H + h;
-      o += p.part_o[cell * p.rank + c] * expf(p.part_m[cell] - mx);
+    const float m = z < ns ? p.part_m[cell] : -1e30f;
+    const float mx = wave_max(m);
+    const float w = z < ns ? expf(m - mx) : 0.f;
+    const float den = wave_sum(z < ns ? p.part_l[cell] * w : 0.f);
+    wz[z] = w;
+    if (z == 0) {
+      float f = 1.0f / den;
+      const T* gate = static_cast<const T*>(p.gate);
+      if (gate) f *= 1.0f / (1.0f + expf(-to_f32(gate[t * p.gate_st + h])));
+      fsh = f;
     }
-    out[t * p.o_st + (int64_t)h * p.o_sh + c] = from_f32<T>(o * f);
+  }
+  __syncthreads();
+  const float f = fsh;
+  T* out = static_cast<T*>(p.out) + t * p.o_st + (int64_t)h * p.o_sh;
+  const int64_t cell0 = (t * p.H + h) * (int64_t)p.rank, zstride = p.tokens * p.H * (int64_t)p.rank;
+  if (p.rank % 4 == 0) {
+    for (int c = 4 * threadIdx.x; c < p.rank; c += 4 * 128) {
+      float4 o = float4{0.f, 0.f, 0.f, 0.f};
+      for (int z = 0; z < ns; ++z) {
+        const float4 v = *reinterpret_cast<const float4*>(p.part_o + z * zstride + cell0 + c);
+        const float w = wz[z];
+        o.x += v.x * w; o.y += v.y * w; o.z += v.z * w; o.w += v.w * w;
+      }
+      out[c] = from_f32<T>(o.x * f); out[c + 1] = from_f32<T>(o.y * f);
+      out[c + 2] = from_f32<T>(o.z * f); out[c + 3] = from_f32<T>(o.w * f);
+    }
+  } else {
+    for (int c = threadIdx.x; c < p.rank; c += 128) {
+      float o = 0.f;
+      for (int z = 0; z < ns; ++z) o += p.part_o[z * zstride + cell0 + c] * wz[z];
+      out[c] = from_f32<T>(o * f);
+    }
   }
 }
 
-template <typename T> inline bool launch_latent_mfma(const LatentAttnParams& p, dim3 grid, size_t lds, hipStream_t st) {
-#define MI355_LM_CASE(N)                                                                                         \
+template <typename T> inline bool launch_latent_mfma(const LatentAttnParams& p, dim3 grid, bool small, hipStream_t st) {
+#define MI355_LM_LAUNCH(N, ROWS_)                                                                                \
   {                                                                                                              \
-    auto kern = latent_window_attention_mfma_kernel<T, N>;                                                       \
+    auto kern = latent_window_attention_mfma_kernel<T, N, ROWS_>;                                                \
+    const size_t lds = lm_lds_bytes(p.rank, p.dr, ROWS_);                                                        \
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, p);                                                       \
+  }
+#define MI355_LM_CASE(N)                 \
+  {                                      \
+    if (small) MI355_LM_LAUNCH(N, 16)    \
+    else MI355_LM_LAUNCH(N, LM_ROWS)     \
   }
   const int tiles = (p.rank + 15) / 16;
   if (tiles <= 4) MI355_LM_CASE(4)
@@ -496,6 +554,7 @@ template <typename T> inline bool launch_latent_mfma(const LatentAttnParams& p, 
   else if (tiles <= 32) MI355_LM_CASE(32)
   else return false;
 #undef MI355_LM_CASE
+#undef MI355_LM_LAUNCH
   return true;
 }
 
@@ -575,14 +634,15 @@ int mi355_latent_window_attention(void* out, const void* qa, const void* qr, con
   if (mfma) {
     const dim3 mgrid((unsigned)num_blocks, (unsigned)((heads + pl.hg - 1) / pl.hg), (unsigned)num_splits);
     bool ok = false;
-    if (dtype == MI355_BF16) ok = launch_latent_mfma<bf16_t>(p, mgrid, pl.lds, (hipStream_t)stream);
-    else ok = launch_latent_mfma<f16_t>(p, mgrid, pl.lds, (hipStream_t)stream);
+    const bool small = blocks == nullptr && pl.hg <= 16;     // one token per run: at most 16 rows per workgroup
+    if (dtype == MI355_BF16) ok = launch_latent_mfma<bf16_t>(p, mgrid, small, (hipStream_t)stream);
+    else ok = launch_latent_mfma<f16_t>(p, mgrid, small, (hipStream_t)stream);
     MI355_REQUIRE(ok, MI355_ERR_UNSUPPORTED, "latent_window_attention: rank %d is not served", rank);
     MI355_CHECK_LAUNCH("latent_window_attention");
     if (num_splits > 1) {
       const dim3 g2((unsigned)tokens, (unsigned)heads);
-      if (dtype == MI355_BF16) hipLaunchKernelGGL((latent_window_merge_kernel<bf16_t>), g2, dim3(64), 0, (hipStream_t)stream, p);
-      else hipLaunchKernelGGL((latent_window_merge_kernel<f16_t>), g2, dim3(64), 0, (hipStream_t)stream, p);
+      if (dtype == MI355_BF16) hipLaunchKernelGGL((latent_window_merge_kernel<bf16_t>), g2, dim3(128), 0, (hipStream_t)stream, p);
+      else hipLaunchKernelGGL((latent_window_merge_kernel<f16_t>), g2, dim3(128), 0, (hipStream_t)stream, p);
       MI355_CHECK_LAUNCH("latent_window_attention (merge)");
     }
     return MI355_OK;

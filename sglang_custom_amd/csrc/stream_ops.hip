@@ -144,7 +144,23 @@ __device__ __forceinline__ float gelu_tanh_f(float z) {
 }
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
-// out[t][i] = gelu_tanh(gate[t][i]) * up[t][i]
+// out[t][i] = gelu_tanh(gate[t][i]) * up[t][i], 16 bytes of each operand per thread (d and the row stride multiples of the
+// vector length, pointers 16-byte aligned)
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_tanh_and_mul_vec_kernel(T* __restrict__ out, const T* __restrict__ gate, const T* __restrict__ up,
+                                                                   int64_t rows, int64_t d, int64_t in_stride) {
+  constexpr int VE = V16<T>::n;
+  const int64_t per_row = d / VE, n = rows * per_row;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = idx / per_row, i = (idx - r * per_row) * VE;
+    const Vec<T, VE> g = ldvec<T, VE>(gate + r * in_stride + i), u = ldvec<T, VE>(up + r * in_stride + i);
+    Vec<T, VE> o;
+#pragma unroll
+    for (int j = 0; j < VE; ++j) o.v[j] = from_f32<T>(gelu_tanh_f(to_f32(g.v[j])) * to_f32(u.v[j]));
+    stvec<T, VE>(out + r * d + i, o);
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void gelu_tanh_and_mul_kernel(T* __restrict__ out, const T* __restrict__ gate, const T* __restrict__ up,
                                                                int64_t rows, int64_t d, int64_t in_stride) {
@@ -239,8 +255,15 @@ int mi355_gelu_tanh_and_mul(void* out, const void* gate, const void* up, int64_t
   if (rows == 0) return MI355_OK;
   const int grid = (int)std::min<int64_t>((rows * d + 255) / 256, 256 * 16);
   MI355_DISPATCH_DTYPE(dtype, "gelu_tanh_and_mul", {
-    hipLaunchKernelGGL((gelu_tanh_and_mul_kernel<T>), dim3(grid), dim3(256), 0, (hipStream_t)stream, (T*)out, (const T*)gate,
-                       (const T*)up, rows, d, in_stride);
+    constexpr int VE = V16<T>::n;
+    if (d % VE == 0 && in_stride % VE == 0 && aligned16(out) && aligned16(gate) && aligned16(up)) {
+      const int vgrid = (int)std::min<int64_t>((rows * (d / VE) + 255) / 256, 256 * 16);
+      hipLaunchKernelGGL((gelu_tanh_and_mul_vec_kernel<T>), dim3(vgrid), dim3(256), 0, (hipStream_t)stream, (T*)out, (const T*)gate,
+                         (const T*)up, rows, d, in_stride);
+    } else {
+      hipLaunchKernelGGL((gelu_tanh_and_mul_kernel<T>), dim3(grid), dim3(256), 0, (hipStream_t)stream, (T*)out, (const T*)gate,
+                         (const T*)up, rows, d, in_stride);
+    }
   });
   MI355_CHECK_LAUNCH("gelu_tanh_and_mul");
   return MI355_OK;
