@@ -298,29 +298,36 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
     j_hi = min(j_hi, j_lo + chunk - 1);
   }
 
-  // ---- queries into LDS: absorbed part as is, rope part rotated in fp32 and rounded, padding zero
-  for (int idx = tid; idx < ROWS * RP; idx += 256) {
-    const int m = idx / RP, r = idx - m * RP;
-    float v = 0.f;
-    if (m < M && r < R) {
-      const int ti = m / nh, hi = m - ti * nh;
-      if (r < rank) {
-        v = to_f32(qa[(int64_t)(t0 + ti) * p.qa_st + (int64_t)(h0 + hi) * p.qa_sh + r]);
-      } else {
-        const int i = r - rank, half = p.rot_dims >> 1;
-        const T* src = qr + (int64_t)(t0 + ti) * p.qr_st + (int64_t)(h0 + hi) * p.qr_sh;
-        if (i >= p.rot_dims) {
-          v = to_f32(src[i]);
-        } else {
-          const int f = i < half ? i : i - half;
-          float sn, cs;
-          sincosf((float)(p0 + ti) * p.inv_freq[f], &sn, &cs);
-          const float u = to_f32(src[f]), w = to_f32(src[f + half]);
-          v = i < half ? u * cs - w * sn : w * cs + u * sn;
-        }
+  // ---- queries into LDS: absorbed part as is, rope part rotated in fp32 and rounded, padding zero.  A wave takes
+  // whole rows (no per-element division); the absorbed part moves as 16-byte vectors when the strides allow it.
+  {
+    const bool qvec = (rank % 8 == 0) && (p.qa_st % 8 == 0) && (p.qa_sh % 8 == 0) && aligned16(qa);
+    const int half = p.rot_dims >> 1;
+    for (int m = wave; m < ROWS; m += 4) {
+      T* dst = Qs + (size_t)m * LD;
+      if (m >= M) {
+        for (int r = 8 * lane; r < RP; r += 512) stvec<T, 8>(dst + r, Vec<T, 8>{});
+        continue;
       }
+      const int ti = m / nh, hi = m - ti * nh;
+      const T* src = qa + (int64_t)(t0 + ti) * p.qa_st + (int64_t)(h0 + hi) * p.qa_sh;
+      if (qvec) {
+        for (int r = 8 * lane; r < rank; r += 512) stvec<T, 8>(dst + r, ldvec<T, 8>(src + r));
+      } else {
+        for (int r = lane; r < rank; r += 64) dst[r] = src[r];
+      }
+      const T* rs = qr + (int64_t)(t0 + ti) * p.qr_st + (int64_t)(h0 + hi) * p.qr_sh;
+      const float pos = (float)(p0 + ti);
+      for (int i = lane; i < half; i += 64) {
+        float sn, cs;
+        sincosf(pos * p.inv_freq[i], &sn, &cs);
+        const float u = to_f32(rs[i]), w = to_f32(rs[i + half]);
+        dst[rank + i] = from_f32<T>(u * cs - w * sn);
+        dst[rank + i + half] = from_f32<T>(w * cs + u * sn);
+      }
+      for (int i = p.rot_dims + lane; i < dr; i += 64) dst[rank + i] = rs[i];
+      for (int r = R + lane; r < RP; r += 64) dst[r] = from_f32<T>(0.f);
     }
-    Qs[(size_t)m * LD + r] = from_f32<T>(v);
   }
 
   // ---- running softmax state of this lane's four rows (rows 16 wave + 4 lg + r), replicated over the 16 lanes
@@ -338,26 +345,44 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
 #pragma unroll
   for (int c = 0; c < NRT; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bool vec_ok = (R % 8 == 0) && aligned16(cache);
-  const int chunks = RP / 8;
   __syncthreads();
 
   for (int64_t j0 = j_lo; j0 <= j_hi; j0 += LM_KB) {
     const int kn = (int)min((int64_t)LM_KB, j_hi - j0 + 1);
-    if (tid < LM_KB) kslot[tid] = tid < kn ? table[j0 + tid] : 0;
-    __syncthreads();
-    for (int idx = tid; idx < LM_KB * chunks; idx += 256) {
-      const int jj = idx / chunks, ch = idx - jj * chunks;
-      Vec<T, 8> v;
-      if (jj < kn && vec_ok && 8 * ch + 8 <= R) {
-        v = ldvec<T, 8>(cache + (int64_t)kslot[jj] * R + 8 * ch);
-      } else {
+    // wave w brings rows w, w + 4, ..: four rows per round, each lane up to two 16-byte pieces of a row, all of a
+    // round's loads issued before the first store; rows past the last key and columns past R are zero
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int r = 8 * ch + e;
-          v.v[e] = (jj < kn && r < R) ? cache[(int64_t)kslot[jj] * R + r] : from_f32<T>(0.f);
+    for (int rb = 0; rb < LM_KB / 4; rb += 4) {
+      Vec<T, 8> v[4][2];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int jj = wave + 4 * (rb + q);
+        const T* row = cache + (int64_t)(jj < kn ? table[j0 + jj] : 0) * R;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int r = 8 * (lane + 64 * e);
+          Vec<T, 8> x{};
+          if (jj < kn && r < R) {
+            if (vec_ok && r + 8 <= R) {
+              x = ldvec<T, 8>(row + r);
+            } else {
+#pragma unroll
+              for (int k = 0; k < 8; ++k)
+                if (r + k < R) x.v[k] = row[r + k];
+            }
+          }
+          v[q][e] = x;
         }
       }
-      stvec<T, 8>(Ks + (size_t)jj * LD + 8 * ch, v);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int jj = wave + 4 * (rb + q);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int r = 8 * (lane + 64 * e);
+          if (r < RP) stvec<T, 8>(Ks + (size_t)jj * LD + r, v[q][e]);
+        }
+      }
     }
     __syncthreads();
     if (wave_has_rows) {
@@ -559,7 +584,8 @@ template <typename T> inline bool launch_latent_mfma(const LatentAttnParams& p, 
 }
 
 inline bool latent_mfma_serves(int dtype, int rank, int dr) {
-  return (dtype == MI355_BF16 || dtype == MI355_F16) && rank <= 512 && lm_lds_bytes(rank, dr) <= 160 * 1024;
+  // (a row of the K tile is at most 2 x 64 pieces of 16 bytes: the loader's two pieces per lane)
+  return (dtype == MI355_BF16 || dtype == MI355_F16) && rank <= 512 && rank + dr <= 1024 && lm_lds_bytes(rank, dr) <= 160 * 1024;
 }
 
 }  // namespace
