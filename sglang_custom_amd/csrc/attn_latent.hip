@@ -255,8 +255,9 @@ inline size_t lm_lds_bytes(int rank, int dr, int rows = LM_ROWS) {
   return 2 * ((size_t)rows * lm_ld(rank, dr) + (size_t)LM_KB * lm_ld(rank, dr) + 4 * 16 * LM_PLD) + sizeof(int) * LM_KB;
 }
 
-// ROWS: query rows the workgroup holds (64; 16 for decode steps of models with at most 16 heads, where only the first
-// wave has rows: the smaller Q tile lets two workgroups share a CU while the other waves still help load the K tiles)
+// ROWS: query rows the workgroup holds (64; 16 or 32 for decode steps of models with at most that many heads, where
+// only the first one or two waves have rows: the smaller Q tile lets two workgroups share a CU while the other waves
+// still help load the K tiles)
 template <typename T, int NRT, int ROWS>
 __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const LatentAttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char sm_raw[];
@@ -559,7 +560,7 @@ __global__ __launch_bounds__(128) void latent_window_merge_kernel(const LatentAt
   }
 }
 
-template <typename T> inline bool launch_latent_mfma(const LatentAttnParams& p, dim3 grid, bool small, hipStream_t st) {
+template <typename T> inline bool launch_latent_mfma(const LatentAttnParams& p, dim3 grid, int rows, hipStream_t st) {
 #define MI355_LM_LAUNCH(N, ROWS_)                                                                                \
   {                                                                                                              \
     auto kern = latent_window_attention_mfma_kernel<T, N, ROWS_>;                                                \
@@ -567,10 +568,11 @@ template <typename T> inline bool launch_latent_mfma(const LatentAttnParams& p, 
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, p);                                                       \
   }
-#define MI355_LM_CASE(N)                 \
-  {                                      \
-    if (small) MI355_LM_LAUNCH(N, 16)    \
-    else MI355_LM_LAUNCH(N, LM_ROWS)     \
+#define MI355_LM_CASE(N)                       \
+  {                                            \
+    if (rows <= 16) MI355_LM_LAUNCH(N, 16)     \
+    else if (rows <= 32) MI355_LM_LAUNCH(N, 32) \
+    else MI355_LM_LAUNCH(N, LM_ROWS)           \
   }
   const int tiles = (p.rank + 15) / 16;
   if (tiles <= 4) MI355_LM_CASE(4)
@@ -660,9 +662,9 @@ int mi355_latent_window_attention(void* out, const void* qa, const void* qr, con
   if (mfma) {
     const dim3 mgrid((unsigned)num_blocks, (unsigned)((heads + pl.hg - 1) / pl.hg), (unsigned)num_splits);
     bool ok = false;
-    const bool small = blocks == nullptr && pl.hg <= 16;     // one token per run: at most 16 rows per workgroup
-    if (dtype == MI355_BF16) ok = launch_latent_mfma<bf16_t>(p, mgrid, small, (hipStream_t)stream);
-    else ok = launch_latent_mfma<f16_t>(p, mgrid, small, (hipStream_t)stream);
+    const int rows = blocks == nullptr ? pl.hg : LM_ROWS;     // one token per run: a workgroup holds at most hg rows
+    if (dtype == MI355_BF16) ok = launch_latent_mfma<bf16_t>(p, mgrid, rows, (hipStream_t)stream);
+    else ok = launch_latent_mfma<f16_t>(p, mgrid, rows, (hipStream_t)stream);
     MI355_REQUIRE(ok, MI355_ERR_UNSUPPORTED, "latent_window_attention: rank %d is not served", rank);
     MI355_CHECK_LAUNCH("latent_window_attention");
     if (num_splits > 1) {

@@ -38,29 +38,43 @@ __device__ __forceinline__ Seg segment_of(int64_t t, const int32_t* tok_req, con
 }
 
 // (x - mean) / sqrt(var + eps) of one row into buf (LDS, D floats); var = mean of squared deviations.  Every thread
-// touches the same elements in all three passes, so buf needs no barrier of its own.
+// touches the same elements in all three passes, so buf needs no barrier of its own.  W = 4: four floats per access
+// (D a multiple of 4, rows 16-byte aligned).
+template <int W>
 __device__ __forceinline__ void ln_row(float* buf, const float* __restrict__ x, int64_t D, float eps, float* red) {
   float s = 0.f;
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-    const float v = x[i];
-    buf[i] = v;
-    s += v;
+  for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+    if constexpr (W == 4) {
+      const float4 v = *reinterpret_cast<const float4*>(x + i);
+      *reinterpret_cast<float4*>(buf + i) = v;
+      s += (v.x + v.y) + (v.z + v.w);
+    } else {
+      const float v = x[i];
+      buf[i] = v;
+      s += v;
+    }
   }
   const float mean = block_sum(s, red) / (float)D;
   float q = 0.f;
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-    const float d = buf[i] - mean;
-    q += d * d;
+  for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      const float d = buf[i + k] - mean;
+      q += d * d;
+    }
   }
   const float var = block_sum(q, red) / (float)D;
   const float inv = 1.0f / sqrtf(var + eps);
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) buf[i] = (buf[i] - mean) * inv;
+  for (int64_t i = W * threadIdx.x; i < D; i += W * blockDim.x) {
+#pragma unroll
+    for (int k = 0; k < W; ++k) buf[i + k] = (buf[i + k] - mean) * inv;
+  }
 }
 
 // One workgroup per token.  h = LN(x[t]) * w;  with `mu`: hs = h + (h_prev - h) * mu, where h_prev is the same
 // quantity of the previous token: zero at position 0, the state row when t opens its segment, else recomputed from
 // x[t - 1].  The last token of every segment leaves its fp32 h in h_last[b] for the commit kernel.
-template <typename T>
+template <typename T, int W>
 __global__ __launch_bounds__(256) void layernorm_shift_kernel(
     T* __restrict__ h_out, T* __restrict__ hs_out, float* __restrict__ h_last, const float* __restrict__ x,
     const T* __restrict__ w, const T* __restrict__ mu, const float* __restrict__ state, const int32_t* __restrict__ req_to_state,
@@ -71,28 +85,46 @@ __global__ __launch_bounds__(256) void layernorm_shift_kernel(
   float* cur = sm;
   float* prv = sm + D;
   const int64_t t = blockIdx.x;
-  ln_row(cur, x + t * D, D, eps, red);
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) cur[i] *= to_f32(w[i]);
+  const int64_t i0 = W * threadIdx.x, step = W * blockDim.x;
+  ln_row<W>(cur, x + t * D, D, eps, red);
   if (mu == nullptr) {
-    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) h_out[t * D + i] = from_f32<T>(cur[i]);
+    for (int64_t i = i0; i < D; i += step) {
+      Vec<T, W> o;
+#pragma unroll
+      for (int k = 0; k < W; ++k) o.v[k] = from_f32<T>(cur[i + k] * to_f32(w[i + k]));
+      stvec<T, W>(h_out + t * D + i, o);
+    }
     return;
   }
   const Seg sg = segment_of(t, tok_req, seg_start, seg_len);
   const int64_t pos = positions[t];
   if (pos == 0) {
-    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) prv[i] = 0.f;
+    for (int64_t i = i0; i < D; i += step)
+#pragma unroll
+      for (int k = 0; k < W; ++k) prv[i + k] = 0.f;
   } else if (sg.first) {
-    const int64_t slot = req_to_state[req_pool_indices[sg.b]];
-    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) prv[i] = state[slot * D + i];
+    const float* srow = state + (int64_t)req_to_state[req_pool_indices[sg.b]] * D;
+    for (int64_t i = i0; i < D; i += step)
+#pragma unroll
+      for (int k = 0; k < W; ++k) prv[i + k] = srow[i + k];
   } else {
-    ln_row(prv, x + (t - 1) * D, D, eps, red);
-    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) prv[i] *= to_f32(w[i]);
+    ln_row<W>(prv, x + (t - 1) * D, D, eps, red);
+    for (int64_t i = i0; i < D; i += step)
+#pragma unroll
+      for (int k = 0; k < W; ++k) prv[i + k] *= to_f32(w[i + k]);
   }
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-    const float h = cur[i];
-    h_out[t * D + i] = from_f32<T>(h);
-    hs_out[t * D + i] = from_f32<T>(h + (prv[i] - h) * to_f32(mu[i]));
-    if (sg.last && h_last != nullptr) h_last[(int64_t)sg.b * D + i] = h;
+  const bool keep = sg.last && h_last != nullptr;
+  for (int64_t i = i0; i < D; i += step) {
+    Vec<T, W> ho, so;
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      const float h = cur[i + k] * to_f32(w[i + k]);
+      ho.v[k] = from_f32<T>(h);
+      so.v[k] = from_f32<T>(h + (prv[i + k] - h) * to_f32(mu[i + k]));
+      if (keep) h_last[(int64_t)sg.b * D + i + k] = h;
+    }
+    stvec<T, W>(h_out + t * D + i, ho);
+    stvec<T, W>(hs_out + t * D + i, so);
   }
 }
 
@@ -204,7 +236,9 @@ int mi355_layernorm_shift(void* h_out, void* hs_out, float* h_last, const float*
   if (tokens == 0) return MI355_OK;
   const size_t lds = (size_t)hidden * 2 * sizeof(float);
   MI355_DISPATCH_DTYPE(dtype, "layernorm_shift", {
-    auto kern = layernorm_shift_kernel<T>;
+    const bool wide = hidden % 4 == 0 && aligned16(x) && aligned16(h_out) && (!hs_out || aligned16(hs_out)) &&
+                      (!state || aligned16(state));
+    auto kern = wide ? layernorm_shift_kernel<T, 4> : layernorm_shift_kernel<T, 1>;
     if (lds > 48 * 1024) (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     hipLaunchKernelGGL(kern, dim3((unsigned)tokens), dim3(256), lds, (hipStream_t)stream, (T*)h_out, (T*)hs_out, h_last, x,
                        (const T*)weight, (const T*)shift, state, req_to_state, req_pool_indices, tok_req, seg_start, seg_len,
