@@ -148,16 +148,29 @@ def load():
     # torch (if used by the caller) must be imported first so that its libamdhip64.so.7 is the
     # one HIP runtime in the process; stream handles are only meaningful within one runtime.
     lib = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+    # a library built for one model family alone (build.build_for) says so in a file beside it: the entry points of the
+    # sources it leaves out raise when called; without that file every declared entry point must be there
+    partial = (not _use_dev) and os.path.exists(path + ".partial")
     for name, (res, args) in list(_SIGNATURES.items()) + (list(_DEV_SIGNATURES.items()) if _use_dev else []):
         fn = getattr(lib, name, None)
         if fn is None:
-            raise Mi355Error(f"{path} does not export {name}")
+            if not partial:
+                raise Mi355Error(f"{path} does not export {name}")
+            setattr(lib, name, _absent(name))
+            continue
         fn.restype = res
         fn.argtypes = args
     if lib.mi355_abi_version() != 1:
         raise Mi355Error("libmi355_hotpath.so ABI version mismatch")
     _lib = lib
     return lib
+
+
+def _absent(name: str):
+    def raise_absent(*_args):
+        raise Mi355Error(f"{name} is not in this partial build of the library (built for one model family): "
+                         "run `python -m sglang_custom_amd.build` for the whole of it")
+    return raise_absent
 
 
 def check(rc: int, what: str):

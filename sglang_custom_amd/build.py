@@ -37,12 +37,53 @@ def _stale(target, deps):
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build(force: bool = False, verbose: bool = False, dev: bool = False) -> str:
+# What one model family needs of the library: a first call in a fresh checkout (bin/trace_run) compiles these and no
+# more.  The result is a PARTIAL library at the usual path, marked by the file PARTIAL_MARK (one source name a line);
+# entry points of the sources left out raise when called (_lib.load), and the next full build() completes it.
+FAMILY_SOURCES = {
+    "Seturax": ["elementwise.hip", "index_ops.hip", "gemm.hip", "gemm_tiled.hip", "stream_ops.hip", "attn_latent.hip"],
+}
+PARTIAL_MARK = LIB + ".partial"
+
+
+def partial_sources():
+    """Sources of the library at LIB if it is a partial build, else None."""
+    if not (os.path.exists(LIB) and os.path.exists(PARTIAL_MARK)):
+        return None
+    with open(PARTIAL_MARK) as f:
+        return [line.strip() for line in f if line.strip()]
+
+
+def build_for(architecture: str, verbose: bool = False) -> str:
+    """The library as far as `architecture` needs it: a complete library that is up to date is used as it is; a missing
+    or stale one is built from the family's sources only (everything, for a family without a list)."""
+    only = FAMILY_SOURCES.get(architecture)
+    if only is None:
+        return build(verbose=verbose)
+    have = partial_sources()
+    deps = [os.path.join(CSRC, s) for s in SOURCES] + HEADERS
+    if os.path.exists(LIB) and have is None and not _stale(LIB, deps):
+        return LIB
+    if have is not None:
+        only = sorted(set(only) | set(have))
+    return build(verbose=verbose, only=only)
+
+
+def build(force: bool = False, verbose: bool = False, dev: bool = False, only=None) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objdir = os.path.join(HERE, "build_dev" if dev else "build")
     os.makedirs(objdir, exist_ok=True)
     srcs = [s for s in SOURCES + (DEV_SOURCES if dev else []) if os.path.exists(os.path.join(CSRC, s))]
+    if only is not None:
+        assert not dev
+        srcs = [s for s in srcs if s in set(only)]
+        if len(srcs) == len(SOURCES):
+            only = None
     lib = LIB_DEV if dev else LIB
+    if not dev and only is None and os.path.exists(PARTIAL_MARK):
+        force_link = True        # a partial library is at the path: link again whatever the time stamps say
+    else:
+        force_link = False
     flags = FLAGS + (["-DMI355_DEV_BUILD"] + os.environ.get("MI355_DEV_EXTRA_FLAGS", "").split() if dev else [])
     objs, procs = [], []
     for s in srcs:
@@ -62,11 +103,20 @@ def build(force: bool = False, verbose: bool = False, dev: bool = False) -> str:
             sys.stderr.write(f"--- hipcc failed on {s} ---\n{out.decode()}\n")
     if failed:
         raise RuntimeError("hipcc compilation failed")
-    if force or procs or _stale(lib, objs):
+    was_partial = partial_sources() if not dev else None
+    if only is not None and (was_partial is None or set(was_partial) != set(srcs)):
+        force_link = True
+    if force or procs or force_link or _stale(lib, objs):
         cmd = [hipcc, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", lib] + objs
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd)
+    if not dev:
+        if only is not None:
+            with open(PARTIAL_MARK, "w") as f:
+                f.write("\n".join(srcs) + "\n")
+        elif os.path.exists(PARTIAL_MARK):
+            os.remove(PARTIAL_MARK)
     return lib
 
 
