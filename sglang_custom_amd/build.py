@@ -55,15 +55,16 @@ def partial_sources():
 
 
 def build_for(architecture: str, verbose: bool = False) -> str:
-    """The library as far as `architecture` needs it: a complete library that is up to date is used as it is; a missing
-    or stale one is built from the family's sources only (everything, for a family without a list)."""
+    """The library as far as `architecture` needs it: a complete library is kept complete (used as it is, or rebuilt
+    whole if a source is newer); where there is none, or a partial one, the family's sources alone are built
+    (everything, for a family without a list)."""
     only = FAMILY_SOURCES.get(architecture)
     if only is None:
         return build(verbose=verbose)
     have = partial_sources()
-    deps = [os.path.join(CSRC, s) for s in SOURCES] + HEADERS
-    if os.path.exists(LIB) and have is None and not _stale(LIB, deps):
-        return LIB
+    if os.path.exists(LIB) and have is None:
+        # a complete library is never replaced by a partial one: it is used, or, if a source is newer, rebuilt whole
+        return build(verbose=verbose)
     if have is not None:
         only = sorted(set(only) | set(have))
     return build(verbose=verbose, only=only)

@@ -256,7 +256,11 @@ CASES = [("float32", 3e-5), ("bfloat16", 6e-2)]
 def test_prefill_decode_portions_and_batches_against_the_oracle(dtype, tol):
     cfg = su.make_config()
     w = su.make_weights(cfg, seed=3)
-    mr = su.build_runner(cfg, w, dtype=dtype, device=DEV, max_total_tokens=64, max_running_requests=3)
+    mr = su.build_runner(cfg, w, dtype=dtype, device=DEV, max_total_tokens=192, max_running_requests=3)
+    # more than 64 rows at once: the prefill-sized GEMM paths, on widths that are multiples of nothing in particular
+    long = su.random_prompts(cfg, [150], seed=4)
+    su.replay_and_compare(mr, cfg, w, long, [[("r0", 150)]], tol)
+    su.replay_and_compare(mr, cfg, w, long, [[("r0", 71)], [("r0", 2)], [("r0", 77)]], tol)
     p = su.random_prompts(cfg, [23], seed=0)
     su.replay_and_compare(mr, cfg, w, p, [[("r0", 23)]], tol)
     su.replay_and_compare(mr, cfg, w, p, [[("r0", 1)] for _ in range(23)], tol)
