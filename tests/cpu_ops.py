@@ -188,7 +188,7 @@ def mla_prefill_assemble_supported(nope, rope, vd, rank, dtype):
 
 
 # ------------------------------------------------------- fp32 residual stream with per-sequence state
-# Restatements of the kernels' contracts (include/mi355_hotpath.h) token by token; they share nothing with the
+# Restatements of what the header says of each kernel (include/mi355_hotpath.h) token by token; they share nothing with the
 # whole-sequence functions of oracle/seturax_ref.py that the tests compare against.
 def _segments(T, tok_req, seg_start, seg_len):
     """(b, first, last) per token."""

@@ -1,7 +1,7 @@
 """Seturax on the CPU: the package's host side (configuration, weight stacking, model wiring, ScheduleBatch /
-ForwardBatch, the KV / request / state pools, TraceReplayer, Scheduler) runs with the CPU checker ops (tests/cpu_ops.py)
+ForwardBatch, the KV / request / state pools, TraceReplayer, Scheduler) runs with the CPU stand-in ops (tests/cpu_ops.py)
 and every logit is compared with the plain whole-sequence implementation in oracle/seturax_ref.py.  The HIP kernels
-have their own file (test_seturax_gpu.py); here the arithmetic is the checker's, the bookkeeping is the product's."""
+have their own file (test_seturax_gpu.py); here the arithmetic is the stand-in's, the bookkeeping is the package's."""
 import pytest
 import torch
 
