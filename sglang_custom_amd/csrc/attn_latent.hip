@@ -248,6 +248,10 @@ __global__ __launch_bounds__(256) void latent_window_attention_kernel(const Late
 // in registers (compile time: 4 accumulators each).
 constexpr int LM_KB = 32;
 constexpr int LM_ROWS = 64;
+// rows a prefill workgroup aims for: 32 (two computing waves) so that two workgroups share a CU and one's K-tile
+// loads overlap the other's products; head counts above 32 take one token of up to 64 heads
+constexpr int LM_PREFILL_ROWS = 32;
+inline int lm_block_tokens(int heads) { return heads >= LM_PREFILL_ROWS ? 1 : LM_PREFILL_ROWS / heads; }
 constexpr int LM_PLD = LM_KB + 8;
 
 inline int lm_ld(int rank, int dr) { return ((rank + dr + 31) & ~31) + 8; }
@@ -616,7 +620,7 @@ int mi355_latent_norms_rope_write(void* cq, void* cache, const void* a, const vo
 
 int mi355_latent_window_attention_block_tokens(int heads, int rank, int rope_dim, int dtype) {
   if (heads <= 0 || rank <= 0 || rope_dim < 0) return 0;
-  if (latent_mfma_serves(dtype, rank, rope_dim)) return heads >= LM_ROWS ? 1 : LM_ROWS / heads;
+  if (latent_mfma_serves(dtype, rank, rope_dim)) return lm_block_tokens(heads);
   const LatentAttnPlan pl = plan_latent_attn(heads, rank, rope_dim);
   return pl.lds <= 160 * 1024 ? pl.bq : 0;
 }
@@ -641,7 +645,7 @@ int mi355_latent_window_attention(void* out, const void* qa, const void* qr, con
   LatentAttnPlan pl = plan_latent_attn(heads, rank, rope_dim);
   if (mfma) {
     pl.hg = std::min(heads, LM_ROWS);
-    pl.bq = heads >= LM_ROWS ? 1 : LM_ROWS / heads;
+    pl.bq = lm_block_tokens(heads);
     pl.kb = LM_KB;
     pl.lds = lm_lds_bytes(rank, rope_dim);
   }
@@ -662,7 +666,7 @@ int mi355_latent_window_attention(void* out, const void* qa, const void* qr, con
   if (mfma) {
     const dim3 mgrid((unsigned)num_blocks, (unsigned)((heads + pl.hg - 1) / pl.hg), (unsigned)num_splits);
     bool ok = false;
-    const int rows = blocks == nullptr ? pl.hg : LM_ROWS;     // one token per run: a workgroup holds at most hg rows
+    const int rows = blocks == nullptr ? pl.hg : pl.hg * pl.bq;     // one token per run: a workgroup holds at most hg rows
     if (dtype == MI355_BF16) ok = launch_latent_mfma<bf16_t>(p, mgrid, rows, (hipStream_t)stream);
     else ok = launch_latent_mfma<f16_t>(p, mgrid, rows, (hipStream_t)stream);
     MI355_REQUIRE(ok, MI355_ERR_UNSUPPORTED, "latent_window_attention: rank %d is not served", rank);
