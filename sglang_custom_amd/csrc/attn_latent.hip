@@ -246,6 +246,24 @@ __global__ __launch_bounds__(256) void latent_window_attention_kernel(const Late
 // registers), P rounded to T and passed through LDS into the A layout of v_mfma_f32_16x16x16, whose B operand -- the
 // value part of the same K tile -- comes from a transposed LDS read.  NRT = 16-column tiles of the value part kept
 // in registers (compile time: 4 accumulators each).
+// Reductions over the 16 lanes that hold one row's scores, on the data-parallel-primitive path of the vector ALU
+// (quad swaps, then the mirror of each half row, then the mirror of the row) instead of LDS permutes.
+template <int CTRL> __device__ __forceinline__ float lm_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float lm_row16_max(float v) {
+  v = fmaxf(v, lm_dpp<0xB1>(v));
+  v = fmaxf(v, lm_dpp<0x4E>(v));
+  v = fmaxf(v, lm_dpp<0x141>(v));
+  return fmaxf(v, lm_dpp<0x140>(v));
+}
+__device__ __forceinline__ float lm_row16_sum(float v) {
+  v += lm_dpp<0xB1>(v);
+  v += lm_dpp<0x4E>(v);
+  v += lm_dpp<0x141>(v);
+  return v + lm_dpp<0x140>(v);
+}
+
 constexpr int LM_KB = 32;
 constexpr int LM_ROWS = 64;
 // rows a prefill workgroup aims for: 32 (two computing waves) so that two workgroups share a CU and one's K-tile
@@ -256,12 +274,11 @@ constexpr int LM_PLD = LM_KB + 8;
 
 inline int lm_ld(int rank, int dr) { return ((rank + dr + 31) & ~31) + 8; }
 inline size_t lm_lds_bytes(int rank, int dr, int rows = LM_ROWS) {
-  return 2 * ((size_t)rows * lm_ld(rank, dr) + (size_t)LM_KB * lm_ld(rank, dr) + 4 * 16 * LM_PLD) + sizeof(int) * LM_KB;
+  return 2 * ((size_t)rows * lm_ld(rank, dr) + (size_t)LM_KB * lm_ld(rank, dr) + (size_t)rows * LM_PLD) + sizeof(float) * 2 * rows;
 }
 
-// ROWS: query rows the workgroup holds (64; 16 or 32 for decode steps of models with at most that many heads, where
-// only the first one or two waves have rows: the smaller Q tile lets two workgroups share a CU while the other waves
-// still help load the K tiles)
+// ROWS: query rows the workgroup holds: 16, 32 or 64 (the smallest that takes the run's tokens x heads); with 16 or 32
+// two workgroups share a CU
 template <typename T, int NRT, int ROWS>
 __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const LatentAttnParams p) {
   extern __shared__ __attribute__((aligned(16))) char sm_raw[];
@@ -271,8 +288,9 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
   const int RP = (R + 31) & ~31, LD = RP + 8;
   T* Qs = reinterpret_cast<T*>(sm_raw);                 // [64][LD]
   T* Ks = Qs + (size_t)ROWS * LD;                       // [32][LD]
-  T* Ps = Ks + (size_t)LM_KB * LD;                      // [4][16][LM_PLD]
-  int* kslot = reinterpret_cast<int*>(Ps + 4 * 16 * LM_PLD);
+  T* Ps = Ks + (size_t)LM_KB * LD;                      // [ROWS][LM_PLD]: the tile's softmax weights, rounded to T
+  float* alpha_s = reinterpret_cast<float*>(Ps + (size_t)ROWS * LM_PLD);   // [ROWS]: this tile's rescale of the running sums
+  float* l_s = alpha_s + ROWS;                                              // [ROWS]: final denominators
   int t0, n;
   if (p.blocks) {
     t0 = p.blocks[2 * blockIdx.x];
@@ -336,19 +354,25 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
   }
 
   // ---- running softmax state of this lane's four rows (rows 16 wave + 4 lg + r), replicated over the 16 lanes
+  // Scores and softmax go by ROWS: wave w owns the 16 rows of row tile w.  The products with V go by COLUMNS: wave w
+  // owns column tiles w CT .. w CT + CT - 1 of the result for every row tile, so that each V fragment is read from LDS
+  // once per workgroup and serves all row tiles; the weights P and the rescale factors cross between the waves in LDS.
+  constexpr int RT = ROWS / 16, CT = NRT / 4;
   const int r0 = 16 * wave;
-  const bool wave_has_rows = r0 < M && r0 < ROWS;
+  const bool wave_has_rows = r0 < ROWS;
   float mrun[4], lrun[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int m = r0 + 4 * lg + r;
     const bool with_sink = split == 0 && m < M;
-    mrun[r] = with_sink ? p.sink[h0 + (m % nh)] : -1e30f;
+    mrun[r] = with_sink ? p.sink[h0 + (m % nh)] * 1.4426950408889634f : -1e30f;     // base-2 units, as the scores
     lrun[r] = with_sink ? 1.0f : 0.0f;
   }
-  f32x4 acc[NRT];
+  f32x4 acc[RT][CT];
 #pragma unroll
-  for (int c = 0; c < NRT; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int c = 0; c < CT; ++c) acc[rt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
   const bool vec_ok = (R % 8 == 0) && aligned16(cache);
   __syncthreads();
 
@@ -417,101 +441,120 @@ __global__ __launch_bounds__(256) void latent_window_attention_mfma_kernel(const
         s0 = Mfma<T>::run(a, *reinterpret_cast<const frag*>(k0row + kc), s0);
         s1 = Mfma<T>::run(a, *reinterpret_cast<const frag*>(k1row + kc), s1);
       }
-      float pr[2][4], alpha[4];
+      // softmax in base 2: exp(x) = 2^(x log2 e), with the scale folded into the factor; the four rows' reductions are
+      // independent chains
+      float pr[2][4], alpha[4], sv[2][4], mx[4];
+      const float sl2 = p.scale * 1.4426950408889634f;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int m = r0 + 4 * lg + r;
         const int64_t pq = p0 + m / nh;
-        float sv[2] = {s0[r], s1[r]};
-        float mx = -INFINITY;
+        const float raw[2] = {s0[r], s1[r]};
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           const int64_t j = j0 + 16 * h + li;
           const bool vis = m < M && j <= j_hi && j <= pq && pq - j < p.window;
-          sv[h] = vis ? sv[h] * p.scale : -INFINITY;
-          mx = fmaxf(mx, sv[h]);
+          sv[h][r] = vis ? raw[h] * sl2 : -INFINITY;
         }
+        mx[r] = fmaxf(sv[0][r], sv[1][r]);
+      }
 #pragma unroll
-        for (int o = 1; o < 16; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-        const float mnew = fmaxf(mrun[r], mx);
-        alpha[r] = expf(mrun[r] - mnew);
-        float sum = 0.f;
+      for (int r = 0; r < 4; ++r) mx[r] = lm_row16_max(mx[r]);
+      float sum[4];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          pr[h][r] = expf(sv[h] - mnew);
-          sum += pr[h][r];
-        }
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o, 64);
-        lrun[r] = lrun[r] * alpha[r] + sum;
+      for (int r = 0; r < 4; ++r) {
+        const float mnew = fmaxf(mrun[r], mx[r]);
+        alpha[r] = exp2f(mrun[r] - mnew);
+        pr[0][r] = exp2f(sv[0][r] - mnew);
+        pr[1][r] = exp2f(sv[1][r] - mnew);
+        sum[r] = pr[0][r] + pr[1][r];
         mrun[r] = mnew;
       }
-      T* pw = Ps + (size_t)wave * 16 * LM_PLD;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) lrun[r] = lrun[r] * alpha[r] + lm_row16_sum(sum[r]);
+      T* pw = Ps + (size_t)r0 * LM_PLD;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         pw[(4 * lg + r) * LM_PLD + li] = from_f32<T>(pr[0][r]);
         pw[(4 * lg + r) * LM_PLD + 16 + li] = from_f32<T>(pr[1][r]);
+        if (li == 0) alpha_s[r0 + 4 * lg + r] = alpha[r];
       }
-      __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    // ---- O += P V on the k = 32 instruction: lane group lg supplies keys 8 lg .. 8 lg + 7 of the tile, as two
+    // transposed reads of four keys each; V = the first `rank` columns of the K tile.  This wave's CT column tiles:
+    // all their reads first, then every row tile's products.
+    {
+      const T* vrow = Ks + (size_t)(8 * lg + (li >> 2)) * LD + 4 * (li & 3) + 16 * CT * wave;
+      typename TrRead<T>::v4 lo[CT], hi[CT];
 #pragma unroll
-      for (int c = 0; c < NRT; ++c)
+      for (int c = 0; c < CT; ++c) {
+        if (16 * (CT * wave + c) < rank) {
+          lo[c] = TrRead<T>::run(vrow + 16 * c);
+          hi[c] = TrRead<T>::run(vrow + 4 * LD + 16 * c);
+        }
+      }
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[c][r] *= alpha[r];
-      // ---- O += P V on the k = 32 instruction: lane group lg supplies keys 8 lg .. 8 lg + 7 of the tile, as two
-      // transposed reads of four keys each; V = the first `rank` columns of the K tile.  Eight column tiles per
-      // round, all sixteen reads issued before the eight products.
-      const frag pa = *reinterpret_cast<const frag*>(pw + li * LM_PLD + 8 * lg);
-      const T* vrow = Ks + (size_t)(8 * lg + (li >> 2)) * LD + 4 * (li & 3);
+      for (int rt = 0; rt < RT; ++rt) {
+        const frag pa = *reinterpret_cast<const frag*>(Ps + (size_t)(16 * rt + li) * LM_PLD + 8 * lg);
+        const f32x4 al = *reinterpret_cast<const f32x4*>(alpha_s + 16 * rt + 4 * lg);
 #pragma unroll
-      for (int c0 = 0; c0 < NRT; c0 += 8) {
-        if (16 * c0 < rank) {
-          typename TrRead<T>::v4 lo[8], hi[8];
+        for (int c = 0; c < CT; ++c) {
+          if (16 * (CT * wave + c) < rank) {
+            typename TrRead<T>::v4 both[2] = {lo[c], hi[c]};
+            f32x4 o = acc[rt][c];
 #pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            if (c0 + u < NRT) {
-              lo[u] = TrRead<T>::run(vrow + 16 * (c0 + u));
-              hi[u] = TrRead<T>::run(vrow + 4 * LD + 16 * (c0 + u));
-            }
-          }
-#pragma unroll
-          for (int u = 0; u < 8; ++u) {
-            if (c0 + u < NRT) {
-              typename TrRead<T>::v4 both[2] = {lo[u], hi[u]};
-              acc[c0 + u] = Mfma<T>::run(pa, __builtin_bit_cast(frag, both), acc[c0 + u]);
-            }
+            for (int r = 0; r < 4; ++r) o[r] *= al[r];
+            acc[rt][c] = Mfma<T>::run(pa, __builtin_bit_cast(frag, both), o);
           }
         }
       }
-      __builtin_amdgcn_wave_barrier();
     }
     __syncthreads();
   }
-  if (!wave_has_rows) return;
-  // ---- epilogue: this lane holds rows 16 wave + 4 lg + r, columns 16 c + li
-  T* out = static_cast<T*>(p.out);
-  const T* gate = static_cast<const T*>(p.gate);
+  // ---- epilogue: the row owners publish the denominators (and, for a key range, the range's maximum and sum); then
+  // every wave writes its columns of all rows: this lane holds rows 16 rt + 4 lg + r, columns 16 (CT wave + c) + li
+  if (wave_has_rows) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int m = r0 + 4 * lg + r;
-    if (m >= M) continue;
-    const int ti = m / nh, hi = m - ti * nh;
-    const int64_t t = t0 + ti;
-    const int h = h0 + hi;
-    if (p.nsplit > 1) {
-      const int64_t cell = ((int64_t)split * p.tokens + t) * p.H + h;
-      if (li == 0) {
+    for (int r = 0; r < 4; ++r) {
+      const int m = r0 + 4 * lg + r;
+      if (li == 0) l_s[m] = lrun[r];
+      if (p.nsplit > 1 && li == 0 && m < M) {
+        const int ti = m / nh, hi = m - ti * nh;
+        const int64_t cell = ((int64_t)split * p.tokens + (t0 + ti)) * p.H + (h0 + hi);
         p.part_m[cell] = mrun[r];
         p.part_l[cell] = lrun[r];
       }
+    }
+  }
+  __syncthreads();
+  T* out = static_cast<T*>(p.out);
+  const T* gate = static_cast<const T*>(p.gate);
 #pragma unroll
-      for (int c = 0; c < NRT; ++c)
-        if (16 * c + li < rank) p.part_o[cell * rank + 16 * c + li] = acc[c][r];
-    } else {
-      float f = 1.0f / lrun[r];
-      if (gate) f *= 1.0f / (1.0f + expf(-to_f32(gate[t * p.gate_st + h])));
+  for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-      for (int c = 0; c < NRT; ++c)
-        if (16 * c + li < rank) out[t * p.o_st + (int64_t)h * p.o_sh + 16 * c + li] = from_f32<T>(acc[c][r] * f);
+    for (int r = 0; r < 4; ++r) {
+      const int m = 16 * rt + 4 * lg + r;
+      if (m >= M) continue;
+      const int ti = m / nh, hi = m - ti * nh;
+      const int64_t t = t0 + ti;
+      const int h = h0 + hi;
+      if (p.nsplit > 1) {
+        const int64_t cell = ((int64_t)split * p.tokens + t) * p.H + h;
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+          const int col = 16 * (CT * wave + c) + li;
+          if (col < rank) p.part_o[cell * rank + col] = acc[rt][c][r];
+        }
+      } else {
+        float f = 1.0f / l_s[m];
+        if (gate) f *= 1.0f / (1.0f + expf(-to_f32(gate[t * p.gate_st + h])));
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+          const int col = 16 * (CT * wave + c) + li;
+          if (col < rank) out[t * p.o_st + (int64_t)h * p.o_sh + col] = from_f32<T>(acc[rt][c][r] * f);
+        }
+      }
     }
   }
 }
@@ -530,7 +573,7 @@ __global__ __launch_bounds__(128) void latent_window_merge_kernel(const LatentAt
     const int64_t cell = ((int64_t)z * p.tokens + t) * p.H + h;
     const float m = z < ns ? p.part_m[cell] : -1e30f;
     const float mx = wave_max(m);
-    const float w = z < ns ? expf(m - mx) : 0.f;
+    const float w = z < ns ? exp2f(m - mx) : 0.f;
     const float den = wave_sum(z < ns ? p.part_l[cell] * w : 0.f);
     wz[z] = w;
     if (z == 0) {
