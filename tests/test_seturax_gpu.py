@@ -226,9 +226,23 @@ def test_window_edges_far_keys_and_the_sink_show(dtype):
             rows[planted, rank:] = ref.rotate_half(k, torch.tensor([p]), 10000.0, dr)[0, 0].to(dtype)
             qr[..., 0] = 8.0
         cache[req_to_token[0].long()] = rows.to(DEV)
+        sink = torch.full((H,), sink_value, device=DEV)
         out = torch.zeros(1, H, rank, dtype=dtype, device=DEV)
         ops().latent_window_attention(qa.to(DEV), qr.to(DEV), cache, out, req_to_token, torch.zeros(1, dtype=torch.int64, device=DEV),
-                                      torch.tensor([p], device=DEV), torch.full((H,), sink_value, device=DEV), inv_freq, dr, window, 1.0)
+                                      torch.tensor([p], device=DEV), sink, inv_freq, dr, window, 1.0)
+        # the same query as the last token of a prompt portion (the three before it ask for nothing in particular): the
+        # run's key range starts earlier than this query's window, so the per-row mask has to cut it
+        n_q = min(4, ops().latent_window_attention_block_tokens(H, rank, dr, dtype))
+        if n_q > 1:
+            qa4 = torch.cat([torch.zeros(n_q - 1, H, rank, dtype=dtype), qa]).to(DEV)
+            qr4 = torch.cat([torch.zeros(n_q - 1, H, dr, dtype=dtype), qr]).to(DEV)
+            out4 = torch.zeros(n_q, H, rank, dtype=dtype, device=DEV)
+            ops().latent_window_attention(qa4, qr4, cache, out4, req_to_token, torch.zeros(1, dtype=torch.int64, device=DEV),
+                                          torch.arange(p - n_q + 1, p + 1, device=DEV), sink, inv_freq, dr, window, 1.0,
+                                          tok_req=torch.zeros(n_q, dtype=torch.int32, device=DEV),
+                                          blocks=torch.tensor([[0, n_q]], dtype=torch.int32, device=DEV))
+            assert (out4[-1].float() - out[0].float()).abs().max() < (1e-5 if dtype == torch.float32 else 1e-2), \
+                "a query answers differently inside a prompt portion"
         return out[0, 0].cpu().double(), rows.double()
 
     tol = 1e-4 if dtype == torch.float32 else 2e-2
@@ -288,6 +302,19 @@ def test_long_decode_across_windows_and_pages(dtype, tol, page_size):
     sched = [[("r0", 40), ("r1", 2)]] + [[("r0", 1), ("r1", 1)] for _ in range(73)] + [[("r0", 1)] for _ in range(77)]
     su.replay_and_compare(mr, cfg, w, p, sched, tol)
     su.replay_and_compare(mr, cfg, w, p, [[("r1", 75)], [("r0", 100)], [("r0", 31)], [("r0", 2)], [("r0", 57)]], tol)
+    assert su.pools_are_whole(mr)
+
+
+@pytest.mark.parametrize("dtype,tol", CASES)
+def test_equal_and_unit_sizes(dtype, tol):
+    """One head, rope width equal to the head width, value width equal to the rank, rank 2, window 1 and a window longer
+    than any prompt, width equal to the vocabulary, one bigram bucket."""
+    layers = [(su.mixer(1, 4, 4, 8, 8, 8, 1), 8), (su.mixer(4, 2, 2, 2, 2, 2, 1000), None)]
+    cfg = su.make_config(width=16, vocab=16, layers=layers, buckets=1, mul_prev=1, mul_cur=1, scale=1.0, logit_scale=1.0)
+    w = su.make_weights(cfg, seed=11)
+    prompts = su.random_prompts(cfg, [14, 5], seed=1)
+    mr = su.build_runner(cfg, w, dtype=dtype, device=DEV, max_total_tokens=32)
+    su.replay_and_compare(mr, cfg, w, prompts, [[("r0", 3), ("r1", 1)], [("r0", 1), ("r1", 1)], [("r0", 10), ("r1", 3)]], tol)
     assert su.pools_are_whole(mr)
 
 
