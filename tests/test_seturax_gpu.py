@@ -345,3 +345,69 @@ def test_greedy_generation_through_the_scheduler(dtype):
     else:
         same = sum(outs[0][k] == outs[1][k] for k in prompts)
         assert same >= len(prompts) - 1
+
+
+def _write_model_folder(folder, cfg, weights):
+    """config.json + model.safetensors (8-byte header length, JSON header, raw little-endian data), written by hand."""
+    import json
+    import struct
+
+    header, blobs, at = {}, [], 0
+    for name, t in weights.items():
+        raw = t.contiguous().view(torch.int16).numpy().tobytes() if t.dtype == torch.bfloat16 else t.contiguous().numpy().tobytes()
+        kind = {torch.bfloat16: "BF16", torch.float32: "F32", torch.int32: "I32"}[t.dtype]
+        header[name] = {"dtype": kind, "shape": list(t.shape), "data_offsets": [at, at + len(raw)]}
+        blobs.append(raw)
+        at += len(raw)
+    head = json.dumps(header).encode()
+    head += b" " * (-len(head) % 8)
+    with open(folder / "model.safetensors", "wb") as f:
+        f.write(struct.pack("<Q", len(head)) + head + b"".join(blobs))
+    with open(folder / "config.json", "w") as f:
+        json.dump(cfg, f)
+
+
+@pytest.mark.parametrize("dtype,tol", CASES)
+def test_command_line_replay_of_a_model_folder(tmp_path, dtype, tol):
+    """bin/trace_run as a user starts it: a model folder on disk, steps on standard input, logits in files; four live
+    requests at most, a pool that the requests' total would not fit into."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    layers = [(su.mixer(6, 16, 8, 16, 32, 24, 11), 96), (su.mixer(3, 8, 4, 12, 20, 16, 64, base=777.0), None)]
+    cfg = su.make_config(width=64, vocab=83, layers=layers, buckets=29, mul_prev=11, mul_cur=5, scale=2.0, logit_scale=0.75)
+    w = su.make_weights(cfg, seed=17)
+    _write_model_folder(tmp_path, cfg, w)
+    prompts = su.random_prompts(cfg, [70, 33, 1, 64, 40], seed=6)
+    sched = [[("r0", 40), ("r1", 2)], [("r0", 1), ("r1", 30), ("r2", 1), ("r3", 7)], [("r0", 29), ("r1", 1), ("r3", 57)],
+             [("r4", 2)], [("r4", 1)], [("r4", 37)]]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    lines, want, at = [], [], {k: 0 for k in prompts}
+    full = {k: ref.forward(cfg, w, p) for k, p in prompts.items()}
+    for n, step in enumerate(sched):
+        entries, rows, end = [], [], []
+        for name, cnt in step:
+            lo, hi = at[name], at[name] + cnt
+            asked = list(range(0, cnt, 3)) + ([cnt - 1] if (cnt - 1) % 3 else [])
+            entries.append({"id": name, "tokens": prompts[name][lo:hi], "want": asked})
+            rows.append(full[name][lo:hi][asked])
+            at[name] = hi
+            if hi == len(prompts[name]):
+                end.append(name)
+        lines.append(json.dumps({"step": n, "entries": entries, "end": end}))
+        want.append(torch.cat(rows))
+    lines.append(json.dumps({"step": len(sched), "entries": [], "end": []}))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(tmp_path), "--dtype", dtype, "--out", str(out),
+                        "--max-tokens", "192"], input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=300, cwd=root)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [x for x in r.stdout.split("\n") if x.startswith("done")] == [f"done {n}" for n in range(len(sched) + 1)]
+    for n, expect in enumerate(want):
+        got = torch.from_numpy(np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(-1, cfg["vocab"]).copy())
+        assert got.shape == expect.shape
+        assert su.rel_err(got, expect) < tol, f"step {n}"
+    assert not (out / f"{len(sched)}.f32").exists()
