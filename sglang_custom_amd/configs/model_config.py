@@ -23,6 +23,9 @@ class ModelConfig:
         if self.architecture == "Seturax":
             self._init_seturax(c, dtype, context_length, quantization)
             return
+        if self.architecture == "Verozen":
+            self._init_verozen(c, dtype, context_length, quantization)
+            return
         self.hidden_size = c["hidden_size"]
         self.num_hidden_layers = c["num_hidden_layers"]
         self.num_attention_heads = c["num_attention_heads"]
@@ -89,6 +92,60 @@ class ModelConfig:
         self.is_encoder_decoder = False
         self.needs_sequence_state = True     # previous token and previous normed rows travel from step to step
         self.latent_kv = [(s["mixer"]["kv_rank"], s["mixer"]["rot_dim"]) for s in layers]
+
+    def _init_verozen(self, c: dict, dtype: str, context_length: Optional[int], quantization: Optional[str]) -> None:
+        """The Verozen design: "layers" lists the layers one by one, {"type": "gla" | "attention" | "retention", "mixer":
+        {...}, "mlp": {"kind": "moe", "expert": {"ff"}, "router": {...}} | null}; widths under "width" / "vocab", the
+        grouped norm under "norm" {"eps", "groups"}, the residual's weight in front of every norm under "postln_alpha",
+        the per-layer token input under "token_side" {"dim"}.  Layers may differ in every size.  Attention layers keep
+        keys and values per token (kv_layer_shapes), the two recurrent mixers one matrix per head and sequence
+        (recurrent_layer_shapes)."""
+        layers = c["layers"]
+        for i, spec in enumerate(layers):
+            if spec["type"] not in ("gla", "attention", "retention"):
+                raise ValueError(f"Verozen layer {i}: unknown mixer type {spec['type']!r}")
+            if spec.get("mlp") is not None and spec["mlp"].get("kind", "moe") != "moe":
+                raise ValueError(f"Verozen layer {i}: unknown feed-forward kind {spec['mlp'].get('kind')!r}")
+            m = spec["mixer"]
+            if spec["type"] == "attention":
+                if m["heads"] % m.get("kv_heads", m["heads"]):
+                    raise ValueError(f"Verozen layer {i}: {m['heads']} query heads over {m['kv_heads']} key heads")
+                if m.get("vdim", m["dim"]) != m["dim"]:
+                    raise ValueError(f"Verozen layer {i}: the values are the keys, so vdim must equal dim")
+            if spec["type"] == "retention" and len(m["decay"]) != m["heads"]:
+                raise ValueError(f"Verozen layer {i}: {len(m['decay'])} decays for {m['heads']} heads")
+        self.layer_specs = layers
+        self.hidden_size = c["width"]
+        self.vocab_size = c["vocab"]
+        self.num_hidden_layers = len(layers)
+        att = [s["mixer"] for s in layers if s["type"] == "attention"]
+        self.num_attention_heads = max([m["heads"] for m in att] or [1])
+        self.num_key_value_heads = max([m.get("kv_heads", m["heads"]) for m in att] or [1])
+        self.head_dim = max([m["dim"] for m in att] or [1])
+        self.v_head_dim = self.head_dim
+        self.intermediate_size = max([s["mlp"]["expert"]["ff"] for s in layers if s.get("mlp")] or [0])
+        self.rms_norm_eps = c["norm"]["eps"]
+        self.norm_groups = int(c["norm"].get("groups", 1))
+        if self.hidden_size % self.norm_groups:
+            raise ValueError(f"Verozen: width {self.hidden_size} is not a multiple of {self.norm_groups} norm groups")
+        self.postln_alpha = float(c.get("postln_alpha", 1.0))
+        side = c.get("token_side")
+        self.token_side_dim = int(side["dim"]) if side else 0
+        self.rope_theta = None
+        self.rope_scaling = None
+        self.tie_word_embeddings = False
+        self.max_position_embeddings = context_length or 131072     # the design fixes no longest sequence
+        self.context_len = self.max_position_embeddings
+        self.quantization = quantization
+        self.dtype = _DTYPES.get(dtype) or torch.bfloat16
+        self.is_encoder_decoder = False
+        self.needs_sequence_state = any(s["type"] != "attention" for s in layers)
+        # per layer (kv heads, key width, value width) of the layers that cache keys and values, None for the others
+        self.kv_layer_shapes = [(s["mixer"].get("kv_heads", s["mixer"]["heads"]), s["mixer"]["dim"], s["mixer"]["dim"])
+                                if s["type"] == "attention" else None for s in layers]
+        # per layer (heads, key width, value width) of the state matrices of the recurrent layers, None for the others
+        self.recurrent_layer_shapes = [(s["mixer"]["heads"], s["mixer"]["dim"], s["mixer"]["vdim"])
+                                       if s["type"] != "attention" else None for s in layers]
 
     @classmethod
     def from_path(cls, model_path: str, **kw) -> "ModelConfig":

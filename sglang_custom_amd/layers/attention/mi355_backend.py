@@ -64,13 +64,16 @@ class Mi355AttnBackend(AttentionBackend):
         # per-layer latent rows (LatentTokenToKVPool): served by forward_latent_window alone, whose only metadata is
         # the list of token runs per workgroup
         self.is_latent_window = hasattr(model_runner.token_to_kv_pool, "widths")
+        # per-layer key / value shapes (LayeredMHATokenToKVPool): served by forward_sigmoid alone, with the same metadata
+        self.is_layered = hasattr(model_runner.token_to_kv_pool, "layer_shapes")
         self.kv_fp8 = getattr(model_runner.token_to_kv_pool, "dtype", None) == torch.float8_e4m3fn
         if self.is_mla:
             # what the split plan counts is workgroups per sequence, one per 16 query heads
             self.num_kv_head = (self.num_head + 15) // 16
         # value width as the pool stores it (an MLA pool's value is the first kv_lora_rank features of
         # its rows); read from the buffer so that any pool with the reference's accessors works
-        self.v_head_dim = model_runner.token_to_kv_pool.get_value_buffer(0).shape[-1]
+        self.v_head_dim = (cfg.v_head_dim if self.is_layered
+                           else model_runner.token_to_kv_pool.get_value_buffer(0).shape[-1])
         self.max_context_len = int(getattr(cfg, "context_len", 0) or self.req_to_token.shape[1])
         sw = getattr(model_runner, "sliding_window_size", None)
         self.sliding_window_size = sw if sw is not None and sw > 0 else None
@@ -135,7 +138,7 @@ class Mi355AttnBackend(AttentionBackend):
     def init_forward_metadata(self, forward_batch):
         ops = get_ops()
         bs = forward_batch.batch_size
-        if self.is_latent_window:
+        if self.is_latent_window or self.is_layered:
             self.forward_metadata = ForwardMetadata()
             self.forward_metadata.latent_blocks = {}
             return
@@ -309,6 +312,24 @@ class Mi355AttnBackend(AttentionBackend):
         return ops.latent_window_attention(
             qa, qr, cache, out, forward_batch.req_to_token_pool.req_to_token, forward_batch.req_pool_indices,
             forward_batch.positions, layer.sink.data, layer.inv_freq, layer.rot_dims, layer.window, layer.scaling, gate=gate,
+            tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq), num_splits=splits)
+
+    # ---- causal attention with sigmoid weights (no softmax) over per-layer key / value buffers ----
+    def forward_sigmoid(self, q, layer, forward_batch, out):
+        """q [T, H, d] normed and rotated -> out [T, H, dv] = sum over visible keys of sigmoid(q.k * scale * temp_h + bias_h) v.
+        The new tokens' keys and values are in the cache already; prefill portions, decode steps and mixed batches are the
+        same launch, told apart only by the list of token runs.  A decode step with few sequences cuts its keys into
+        ranges whose partial sums a second launch adds (the weights are not normalised, so partial sums simply add)."""
+        ops = get_ops()
+        k_cache, v_cache = forward_batch.token_to_kv_pool.get_kv_buffer(layer.layer_id)
+        bq = ops.sigmoid_attention_block_tokens(layer.tp_q_head_num, layer.tp_k_head_num, q.dtype)
+        splits = 1
+        if forward_batch.forward_mode.is_decode() and forward_batch.seq_lens_cpu is not None:
+            splits = ops.sigmoid_attention_splits(q.shape[0], layer.tp_q_head_num, layer.tp_k_head_num,
+                                                  int(forward_batch.seq_lens_cpu.max()), q.dtype)
+        return ops.sigmoid_attention(
+            q, k_cache, v_cache, out, forward_batch.req_to_token_pool.req_to_token, forward_batch.req_pool_indices,
+            forward_batch.positions, layer.temp.data, layer.bias.data, layer.scaling,
             tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq), num_splits=splits)
 
     def _windowed(self, layer) -> bool:

@@ -1,0 +1,76 @@
+"""LinearRecurrence: the per-layer hand-off to the recurrence kernel for mixers that keep one matrix per head and
+sequence instead of keys and values per token (no counterpart in the reference, whose models keep nothing but KV):
+
+    S_t = diag(a_t) S_{t-1} + k_t v_t^T          S [key width, value width], fp32, zero before position 0
+    o_t = S_t^T (q_t * q_scale)
+
+with the decay a_t either per key channel and token, a_t = sigmoid(z_t + b)^(1 / tau) from gate logits z (gated linear
+attention), or one fixed number per head (retention).  The matrices live in the sequence-state pool
+(SequenceStatePool.matrices[layer]); a step reads a sequence's matrix (or starts from zero at position 0), runs the
+step's tokens of that sequence through it and writes it back, so prefill portions, decode steps and mixed batches are
+the same launch.  Decays, their logarithms and the state are fp32 in every dtype.
+
+HeadNormGate: the recurrence's fp32 output per head divided by its root mean square (times a weight shared by the heads,
+if there is one), times silu(gate), in the activation dtype for the output projection."""
+from typing import Optional
+
+import torch
+from torch import nn
+
+from ..ops_backend import get_ops
+from .rotary_embedding import pair_inv_freq
+
+
+class LinearRecurrence(nn.Module):
+    def __init__(self, num_heads: int, key_dim: int, value_dim: int, layer_id: int, device, q_scale: float = 1.0,
+                 head_decay=None, tau: float = 1.0):
+        super().__init__()
+        self.num_heads, self.key_dim, self.value_dim, self.layer_id = num_heads, key_dim, value_dim, layer_id
+        self.q_scale, self.tau = float(q_scale), float(tau)
+        assert head_decay is None or len(head_decay) == num_heads
+        self.register_buffer("head_decay", None if head_decay is None else
+                             torch.tensor(list(head_decay), dtype=torch.float32, device=device), persistent=False)
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, forward_batch, gate_logits=None, gate_bias=None):
+        """q, k [T, H, dk], v [T, H, dv] (any token stride) -> fp32 [T, H, dv]."""
+        st = forward_batch.seq_state
+        out = torch.empty((q.shape[0], self.num_heads, self.value_dim), dtype=torch.float32, device=q.device)
+        get_ops().linear_recurrence(q, k, v, out, st.pool.matrices[self.layer_id], st.req_to_state, st.req_pool_indices,
+                                    forward_batch.positions, self.q_scale, gate_logits=gate_logits, gate_bias=gate_bias,
+                                    tau=self.tau, head_decay=self.head_decay, **st.segments())
+        return out
+
+
+class HeadNormGate(nn.Module):
+    def __init__(self, value_dim: int, eps: float, dtype, device, with_weight: bool):
+        super().__init__()
+        self.eps = float(eps)
+        self.out_dtype = dtype
+        self.weight = (nn.Parameter(torch.ones(value_dim, dtype=dtype, device=device), requires_grad=False)
+                       if with_weight else None)
+
+    def forward(self, o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+        """o fp32 [T, H, dv], gate [T, H * dv] logits (row-strided) -> [T, H * dv]."""
+        return get_ops().head_rmsnorm_gate(o, self.weight.data if self.weight is not None else None, gate, self.eps,
+                                           self.out_dtype)
+
+
+class HeadNormRope(nn.Module):
+    """Per token and head: an optional RMS norm over the head's features with a weight shared by the heads, then a
+    rotation of the first rot_dims features by position * base^(-2 i / rot_dims) (feature 2 i with 2 i + 1 when
+    `interleaved`, else i with i + rot_dims / 2; angles in fp32 from the position, no table), then a scale.  One
+    launch; the result goes to a new tensor or straight into cache rows."""
+
+    def __init__(self, head_dim: int, rot_dims: int, rot_base: float, interleaved: bool, eps: float, dtype, device,
+                 with_norm: bool, scale: float = 1.0):
+        super().__init__()
+        assert 0 <= rot_dims <= head_dim and rot_dims % 2 == 0
+        self.head_dim, self.rot_dims, self.interleaved, self.eps, self.scale = head_dim, rot_dims, interleaved, float(eps), float(scale)
+        self.weight = nn.Parameter(torch.ones(head_dim, dtype=dtype, device=device), requires_grad=False) if with_norm else None
+        self.register_buffer("inv_freq", pair_inv_freq(rot_base, rot_dims).to(device), persistent=False)
+
+    def forward(self, src: torch.Tensor, positions: torch.Tensor, out_dtype, cache: Optional[torch.Tensor] = None,
+                loc: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """src [T, H, d] (any token stride) -> [T, H, d] of out_dtype, or written to cache[loc[t]] when a cache is given."""
+        return get_ops().head_norm_rope(src, self.weight.data if self.weight is not None else None, self.eps, positions,
+                                        self.inv_freq, self.rot_dims, self.interleaved, self.scale, out_dtype, cache=cache, loc=loc)

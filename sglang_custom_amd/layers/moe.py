@@ -1,0 +1,53 @@
+"""Mixture of experts with a grouped top-k router (the role of the reference's python/sglang/srt/layers/moe/: topk.py
+grouped_topk / biased_grouped_topk and fused_moe_triton/layer.py FusedMoE, re-done for this package's kernels).
+
+  GroupedTopKRouter   scores s = sigmoid(x W_r^T) in fp32.  Selection runs on s + correction; experts form `n_groups`
+                      equal groups of neighbours, a group scores the sum of its two largest selection scores, only
+                      experts of the `keep_groups` best groups can be chosen (the others count as -inf), the `top`
+                      largest are taken.  Weights: the chosen experts' s (without the correction) over their sum
+                      (+ 1e-20), times `scale`.
+  GroupedExperts      expert e: down_e(act(up_e(h))), act = erf-GELU.  Tokens are sorted by expert on the device into
+                      blocks of `block` rows that belong to one expert each (ops.moe_align); two grouped GEMMs run over
+                      the blocks (the first gathers its rows and applies the activation in its epilogue); the weighted
+                      sum over a token's experts is left to the norm kernel that consumes it
+                      (GroupRMSNorm.forward(rows=, coef=)), in a fixed order.  Nothing is read back to the host."""
+from typing import Tuple
+
+import torch
+from torch import nn
+
+from ..ops_backend import get_ops
+
+
+class GroupedTopKRouter(nn.Module):
+    def __init__(self, hidden: int, num_experts: int, top: int, n_groups: int, keep_groups: int, scale: float, device):
+        super().__init__()
+        assert num_experts % n_groups == 0 and 1 <= keep_groups <= n_groups and 1 <= top <= num_experts // n_groups * keep_groups
+        self.num_experts, self.top, self.n_groups, self.keep_groups, self.scale = num_experts, top, n_groups, keep_groups, float(scale)
+        # fp32 whatever the model dtype: the router's logits are computed in fp32 from the fp32 residual stream
+        self.weight = nn.Parameter(torch.zeros(num_experts, hidden, dtype=torch.float32, device=device), requires_grad=False)
+        self.correction = nn.Parameter(torch.zeros(num_experts, dtype=torch.float32, device=device), requires_grad=False)
+
+    def forward(self, x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        """x fp32 [T, D] -> (expert ids int32 [T, top], weights fp32 [T, top])."""
+        ops = get_ops()
+        logits = ops.linear(x, self.weight.data)
+        return ops.moe_route_grouped(logits, self.correction.data, self.top, self.n_groups, self.keep_groups, self.scale)
+
+
+class GroupedExperts(nn.Module):
+    def __init__(self, hidden: int, ff: int, num_experts: int, dtype, device, activation: str = "gelu_erf"):
+        super().__init__()
+        assert activation == "gelu_erf"
+        self.num_experts, self.hidden, self.ff = num_experts, hidden, ff
+        self.w_up = nn.Parameter(torch.zeros(num_experts, ff, hidden, dtype=dtype, device=device), requires_grad=False)
+        self.w_down = nn.Parameter(torch.zeros(num_experts, hidden, ff, dtype=dtype, device=device), requires_grad=False)
+
+    def forward(self, h: torch.Tensor, expert_ids: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        """h [T, D], expert_ids int32 [T, top] -> (y [P, D], rows int32 [T, top]): y[rows[t, j]] is the output of token
+        t's j-th expert; P >= T * top counts the padding of the experts' blocks."""
+        ops = get_ops()
+        plan = ops.moe_align(expert_ids, self.num_experts)
+        a = ops.moe_grouped_linear(h, self.w_up.data, plan, gather=True, gelu=True)
+        y = ops.moe_grouped_linear(a, self.w_down.data, plan, gather=False, gelu=False)
+        return y, plan.rows

@@ -188,3 +188,9 @@ def rotate_half_inv_freq(base: float, dims: int) -> torch.Tensor:
     cos / sin table: nothing bounds the position."""
     i = torch.arange(max(dims // 2, 1), dtype=torch.float64)
     return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / max(dims, 1)).to(torch.float32)
+
+
+def pair_inv_freq(base: float, dims: int) -> torch.Tensor:
+    """The same frequencies for a rotation in either pairing (feature 2 i with 2 i + 1, or i with i + dims / 2): which
+    features form pair i is the kernel's business, f_i is not."""
+    return rotate_half_inv_freq(base, dims)

@@ -202,19 +202,26 @@ class MLATokenToKVPool:
 
 class SequenceStatePool:
     """State that a sequence carries from one step to the next, for models that have such (no counterpart in the
-    reference, whose models keep nothing but KV): per slot the last token id and, per layer, one fp32 row of the
-    model's width (the previous token's normed input of a token-shift layer).  A request holds one slot from its
-    first prefill portion until it finishes or is retracted; what a freed slot holds is never read again, because a
-    sequence's first token (position 0) takes no state.  Slot 0 is never handed out."""
+    reference, whose models keep nothing but KV): per slot the last token id, per layer one fp32 row of the
+    model's width (the previous token's normed input of a token-shift layer) and, for layers with a linear
+    recurrence, one fp32 matrix per head ([heads, key width, value width], `matrices[layer]`; layers may differ).
+    A request holds one slot from its first prefill portion until it finishes or is retracted; what a freed slot
+    holds is never read again, because a sequence's first token (position 0) takes no state.  Slot 0 is never
+    handed out."""
 
-    def __init__(self, size: int, layer_num: int, hidden: int, device: str):
+    def __init__(self, size: int, layer_num: int, hidden: int, device: str, matrices: Optional[dict] = None):
         self.size = size
         self.layer_num = layer_num
         self.hidden = hidden
         self.device = device
         self.rows = torch.zeros((layer_num, size + 1, hidden), dtype=torch.float32, device=device)
         self.prev_token = torch.zeros(size + 1, dtype=torch.int32, device=device)
+        self.matrices = {layer: torch.zeros((size + 1, h, dk, dv), dtype=torch.float32, device=device)
+                         for layer, (h, dk, dv) in (matrices or {}).items()}
         self.free_slots = list(range(1, size + 1))
+
+    def get_state_size_bytes(self) -> int:
+        return self.rows.numel() * 4 + sum(m.numel() * 4 for m in self.matrices.values())
 
     def available_size(self) -> int:
         return len(self.free_slots)
@@ -258,3 +265,34 @@ class LatentTokenToKVPool:
 
     def get_kv_buffer(self, layer_id: int):
         return self.get_key_buffer(layer_id), self.get_value_buffer(layer_id)
+
+
+class LayeredMHATokenToKVPool:
+    """Keys and values per token for models whose layers differ: layer l has its own [size + page_size, heads_l, d_l]
+    key buffer and [size + page_size, heads_l, dv_l] value buffer, or none at all (shapes[l] is None: a layer that
+    keeps no keys, e.g. one with a recurrent mixer).  Slot 0 is the sink row of padded tokens, as in the other
+    pools; one slot index serves every layer."""
+
+    def __init__(self, size: int, page_size: int, dtype: torch.dtype, shapes: List[Optional[Tuple[int, int, int]]], device: str):
+        self.size = size
+        self.page_size = page_size
+        self.dtype = dtype
+        self.store_dtype = dtype
+        self.layer_shapes = list(shapes)
+        self.layer_num = len(shapes)
+        self.device = device
+        rows = size + page_size
+        self.k_buffer = [None if s is None else torch.zeros((rows, s[0], s[1]), dtype=dtype, device=device) for s in shapes]
+        self.v_buffer = [None if s is None else torch.zeros((rows, s[0], s[2]), dtype=dtype, device=device) for s in shapes]
+
+    def get_kv_size_bytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self.k_buffer + self.v_buffer if b is not None)
+
+    def get_key_buffer(self, layer_id: int) -> torch.Tensor:
+        return self.k_buffer[layer_id]
+
+    def get_value_buffer(self, layer_id: int) -> torch.Tensor:
+        return self.v_buffer[layer_id]
+
+    def get_kv_buffer(self, layer_id: int):
+        return self.k_buffer[layer_id], self.v_buffer[layer_id]

@@ -16,6 +16,7 @@ from ..layers.sampler import Sampler
 from ..mem_cache.allocator import PagedTokenToKVPoolAllocator, TokenToKVPoolAllocator
 from ..mem_cache.memory_pool import (
     LatentTokenToKVPool,
+    LayeredMHATokenToKVPool,
     MHATokenToKVPool,
     MLATokenToKVPool,
     ReqToTokenPool,
@@ -120,7 +121,10 @@ class ModelRunner:
         self.kv_cache_dtype = torch.float8_e4m3fn if kvd == "fp8_e4m3" else self.dtype
         mla = getattr(cfg, "is_mla", False)
         latent = getattr(cfg, "latent_kv", None)     # per-layer (rank, rope width) of a latent cache with unequal layers
-        if latent is not None:
+        layered = getattr(cfg, "kv_layer_shapes", None)   # per-layer (kv heads, key width, value width) or None per layer
+        if layered is not None:
+            cell = max(1, sum(h * (dk + dv) for h, dk, dv in filter(None, layered))) * torch.finfo(self.kv_cache_dtype).bits // 8
+        elif latent is not None:
             cell = sum(r + d for r, d in latent) * torch.finfo(self.kv_cache_dtype).bits // 8
         elif mla:
             # one latent row per token and layer (model_runner.py:950-957)
@@ -143,7 +147,11 @@ class ModelRunner:
         page = max(1, int(getattr(sa, "page_size", 1) or 1))
         # whole pages only (model_runner.py:1101-1106 rounds the same way)
         self.max_total_num_tokens = self.max_total_num_tokens // page * page
-        if latent is not None:
+        if layered is not None:
+            if self.kv_cache_dtype != self.dtype:
+                raise ValueError("a cache with per-layer shapes is stored in the model dtype")
+            self.token_to_kv_pool = LayeredMHATokenToKVPool(self.max_total_num_tokens, page, self.kv_cache_dtype, layered, self.device)
+        elif latent is not None:
             if self.kv_cache_dtype != self.dtype:
                 raise ValueError("a latent cache with per-layer widths is stored in the model dtype")
             self.token_to_kv_pool = LatentTokenToKVPool(self.max_total_num_tokens, page, self.kv_cache_dtype, latent, self.device)

@@ -323,3 +323,171 @@ def latent_window_attention(qa, qr, cache, out, req_to_token, req_pool_indices, 
             out[t] = o.to(out.dtype)
     assert bool(covered.all()), "the runs do not cover every token"
     return out
+
+
+# ------------------------------------------------------- post-norm stream, linear recurrences, sigmoid attention, mixture
+# Token-by-token restatements of what the header says of each kernel; they share nothing with the whole-sequence
+# functions of oracle/verozen_ref.py that the tests compare against.
+from types import SimpleNamespace
+
+
+def scaled_add_group_rmsnorm(x, branch, alpha, weight, groups, eps, rows=None, coef=None, inplace=True):
+    T, D = x.shape
+    s = alpha * x
+    if branch is not None:
+        if rows is None:
+            s = s + branch.float()
+        else:
+            for t in range(T):
+                for j in range(rows.shape[1]):
+                    s[t] += float(coef[t, j]) * branch[int(rows[t, j])].float()
+    part = s.view(T, groups, D // groups)
+    n = (part / torch.sqrt((part * part).mean(-1, keepdim=True) + eps)).reshape(T, D) * weight.float()
+    if inplace:
+        x.copy_(n)
+        return x if weight.dtype == torch.float32 else n.to(weight.dtype)
+    return n.to(weight.dtype)
+
+
+def rmsnorm_residual_add(x, y, weight, eps):
+    y = y.float()
+    x.add_(y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps) * weight.float())
+    return x if weight.dtype == torch.float32 else x.to(weight.dtype)
+
+
+def head_norm_rope(src, weight, eps, positions, inv_freq, rot_dims, interleaved, scale, out_dtype, cache=None, loc=None):
+    T, H, d = src.shape
+    out = torch.empty((T, H, d), dtype=torch.float32)
+    for t in range(T):
+        v = src[t].float()
+        if weight is not None:
+            v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight.float()
+        if rot_dims:
+            ang = float(positions[t]) * inv_freq[: rot_dims // 2].float()
+            c, s = torch.cos(ang), torch.sin(ang)
+            r = v.clone()
+            if interleaved:
+                a, b = v[:, 0:rot_dims:2], v[:, 1:rot_dims:2]
+                r[:, 0:rot_dims:2], r[:, 1:rot_dims:2] = a * c - b * s, b * c + a * s
+            else:
+                a, b = v[:, : rot_dims // 2], v[:, rot_dims // 2: rot_dims]
+                r[:, : rot_dims // 2], r[:, rot_dims // 2: rot_dims] = a * c - b * s, b * c + a * s
+            v = r
+        out[t] = v * scale
+    if cache is not None:
+        cache[loc.long()] = out.to(cache.dtype)
+        return cache
+    return out.to(out_dtype)
+
+
+def linear_recurrence(q, k, v, out, state, req_to_state, req_pool_indices, positions, q_scale, gate_logits=None, gate_bias=None,
+                      tau=1.0, head_decay=None, tok_req=None, seg_start=None, seg_len=None):
+    T, H, dk = q.shape
+    S = None
+    for t, (b, first, last) in enumerate(_segments(T, tok_req, seg_start, seg_len)):
+        slot = int(req_to_state[int(req_pool_indices[b])])
+        if first:
+            S = torch.zeros_like(state[slot]) if int(positions[t]) == 0 else state[slot].clone()
+        if gate_logits is not None:
+            z = gate_logits[t].float() + (gate_bias.float() if gate_bias is not None else 0.0)
+            a = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(H, dk)
+        else:
+            a = head_decay.float()[:, None].expand(H, dk)
+        S = a[:, :, None] * S + k[t].float()[:, :, None] * v[t].float()[:, None, :]
+        out[t] = torch.einsum("hkv,hk->hv", S, q[t].float() * q_scale)
+        if last:
+            state[slot] = S
+    return out
+
+
+def head_rmsnorm_gate(o, weight, gate, eps, out_dtype):
+    T, H, dv = o.shape
+    n = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps)
+    if weight is not None:
+        n = n * weight.float()
+    g = gate.float().reshape(T, H, dv)
+    return (n * g * torch.sigmoid(g)).reshape(T, H * dv).to(out_dtype)
+
+
+def sigmoid_attention_block_tokens(heads, kv_heads, dtype):
+    return 3
+
+
+def sigmoid_attention_splits(tokens, heads, kv_heads, max_len, dtype):
+    return 1
+
+
+def sigmoid_attention(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, temp, bias, scale, tok_req=None,
+                      blocks=None, num_splits=1):
+    T, H, d = q.shape
+    G = k_cache.shape[1]
+    covered = torch.zeros(T, dtype=torch.bool)
+    runs = [(t, 1) for t in range(T)] if blocks is None else [(int(a), int(n)) for a, n in blocks.tolist()]
+    for t0, n in runs:
+        for t in range(t0, t0 + n):
+            assert not covered[t]
+            covered[t] = True
+            b = t if tok_req is None else int(tok_req[t])
+            assert blocks is None or int(tok_req[t0]) == b, "a run crosses two sequences"
+            slots = req_to_token[int(req_pool_indices[b]), : int(positions[t]) + 1].long()
+            kk, vv = k_cache[slots].float(), v_cache[slots].float()             # [n, G, d]
+            for h in range(H):
+                g = h // (H // G)
+                s = (kk[:, g] @ q[t, h].float()) * scale * float(temp[h]) + float(bias[h])
+                out[t, h] = (torch.sigmoid(s) @ vv[:, g]).to(out.dtype)
+    assert bool(covered.all()), "the runs do not cover every token"
+    return out
+
+
+def moe_route_grouped(logits, correction, top, n_groups, keep_groups, scale):
+    T, E = logits.shape
+    per = E // n_groups
+    s = torch.sigmoid(logits.float())
+    c = s + correction.float()
+    ids = torch.empty((T, top), dtype=torch.int32)
+    w = torch.empty((T, top), dtype=torch.float32)
+    for t in range(T):
+        gs = c[t].view(n_groups, per).topk(min(2, per), dim=-1).values.sum(-1)
+        kept = set(sorted(range(n_groups), key=lambda g: (-float(gs[g]), g))[:keep_groups])
+        order = sorted((e for e in range(E) if e // per in kept), key=lambda e: (-float(c[t, e]), e))[:top]
+        ids[t] = torch.tensor(order, dtype=torch.int32)
+        sel = s[t, order]
+        w[t] = sel / (sel.sum() + 1e-20) * scale
+    return ids, w
+
+
+def moe_align(expert_ids, num_experts, block=4):
+    T, top = expert_ids.shape
+    flat = expert_ids.reshape(-1).tolist()
+    src, tiles = [], []
+    rows = torch.empty(T * top, dtype=torch.int32)
+    for e in range(num_experts):
+        mine = [i for i, x in enumerate(flat) if x == e]
+        for n, i in enumerate(mine):
+            rows[i] = len(src) + n
+        pad = (-len(mine)) % block
+        tiles += [e] * ((len(mine) + pad) // block)
+        src += [i // top for i in mine] + [-1] * pad
+    return SimpleNamespace(src_row=torch.tensor(src, dtype=torch.int32), rows=rows.view(T, top),
+                           tile_expert=torch.tensor(tiles, dtype=torch.int32), n_tiles=len(tiles), block=block,
+                           padded=len(src))
+
+
+def moe_grouped_linear(x, w, plan, gather, gelu):
+    out = torch.zeros((plan.padded, w.shape[1]), dtype=x.dtype)
+    for p in range(plan.padded):
+        r = int(plan.src_row[p])
+        if r < 0:
+            continue
+        e = int(plan.tile_expert[p // plan.block])
+        y = (x[r] if gather else x[p]).float() @ w[e].float().T
+        if gelu:
+            y = 0.5 * y * (1.0 + torch.erf(y * 0.7071067811865476))
+        out[p] = y.to(x.dtype)
+    return out
+
+
+def gelu_tanh_mul_rows(gate, table, ids, col_off):
+    z = gate.float()
+    g = 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z * z * z)))
+    return (g * table[ids.long(), col_off: col_off + gate.shape[1]].float()).to(gate.dtype)
