@@ -702,6 +702,82 @@ int mi355_latent_window_attention(void* out, const void* qa, const void* qr, con
                                   int64_t req_to_token_stride, int heads, int rank, int rope_dim, int rot_dims, int window,
                                   float scale, int num_splits, float* split_scratch, int64_t tokens, int dtype, void* stream);
 
+/* ---- a 32-bit residual stream that is normed AFTER every residual sum ------------------------------
+ * mi355_scaled_add_group_rmsnorm: y = N(alpha * x[t] + branch(t)) * weight, N = RMS norm over `groups` equal consecutive
+ *   parts of the row (each divided by sqrt(mean(part^2) + eps)); branch(t) is branch[t] (rows null), the sum over
+ *   j < n_branch of coef[t][j] * branch[rows[t][j]] in that order, or nothing (branch null).  y goes to x_out (fp32; may be
+ *   x itself) and / or h_out (T); either may be null.
+ * mi355_rmsnorm_residual_add: x[t] += y[t] / sqrt(mean(y[t]^2) + eps) * weight in place; h_out (T, may be null) = the new x.
+ * mi355_head_norm_rope: per (token, head) row of src [tokens, heads, head_dim] (strided): optional RMS norm with
+ *   `weight` [head_dim] (null: none), then the first rot_dims features rotated by angle position * inv_freq[i], feature
+ *   2i with 2i + 1 (interleaved) or i with i + rot_dims / 2, (a, b) -> (a cos - b sin, b cos + a sin), then times scale.
+ *   Row t goes to out row loc[t] (loc null: t); out_dtype is dtype or MI355_F32.
+ * mi355_head_rmsnorm_gate: out[t][h] = o[t][h] / sqrt(mean(o[t][h]^2) + eps) (* weight [value_dim] unless null)
+ *   * silu(gate[t * gate_stride + h * value_dim + .]), o fp32 [tokens, heads, value_dim] contiguous, out T contiguous.
+ * mi355_gelu_tanh_mul_rows: out[r][i] = gelu_tanh(gate[r][i]) * table[ids[r]][col_off + i]. */
+int mi355_scaled_add_group_rmsnorm(float* x_out, void* h_out, const float* x, const void* branch, int64_t branch_stride,
+                                   const int32_t* rows, const float* coef, int n_branch, float alpha, const void* weight,
+                                   int64_t tokens, int64_t hidden, int groups, float eps, int dtype, void* stream);
+int mi355_rmsnorm_residual_add(float* x, void* h_out, const void* y, int64_t y_stride, const void* weight, int64_t tokens,
+                               int64_t hidden, float eps, int dtype, void* stream);
+int mi355_head_norm_rope(void* out, const void* src, const void* weight, const int64_t* positions, const int64_t* loc,
+                         const float* inv_freq, int64_t tokens, int heads, int head_dim, int64_t src_token_stride,
+                         int64_t src_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t out_rows, int rot_dims,
+                         int interleaved, float scale, float eps, int dtype, int out_dtype, void* stream);
+int mi355_head_rmsnorm_gate(void* out, const float* o, const void* weight, const void* gate, int64_t gate_stride, int64_t tokens,
+                            int heads, int value_dim, float eps, int dtype, void* stream);
+int mi355_gelu_tanh_mul_rows(void* out, const void* gate, int64_t gate_stride, const void* table, int64_t table_rows,
+                             int64_t table_stride, int64_t col_off, const int64_t* ids, int64_t rows, int64_t d, int dtype,
+                             void* stream);
+
+/* ---- linear recurrence with one fp32 matrix per (sequence, head) ------------------------------------
+ * For every sequence b of the step (tokens seg_start[b] .. + seg_len[b]; both null: token b alone), head h:
+ *   S = state[slot(b)][h] ([key_dim, value_dim] fp32; zero instead when the sequence's first token of the step is at
+ *   position 0);  per token  S = diag(a) S + k v^T,  out[t][h] = S^T (q * q_scale);  state[slot(b)][h] = S at the end.
+ *   a[i] = exp(logsigmoid(gate_logits[t][h * key_dim + i] + gate_bias[.]) / tau) (gate_bias of v's type, may be null), or
+ *   head_decay[h] when gate_logits is null.  q, k [tokens, heads, key_dim] of qk_dtype (v_dtype or fp32), v
+ *   [tokens, heads, value_dim], token strides given; out fp32 [tokens, heads, value_dim] contiguous.  key_dim <= 256. */
+int mi355_linear_recurrence(float* out, float* state, const void* q, const void* k, const void* v, const float* gate_logits,
+                            const void* gate_bias, const float* head_decay, const int32_t* req_to_state,
+                            const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len,
+                            const int64_t* positions, int64_t batch, int heads, int key_dim, int value_dim, int64_t q_token_stride,
+                            int64_t k_token_stride, int64_t v_token_stride, int64_t gate_token_stride, float q_scale, float tau,
+                            int qk_dtype, int v_dtype, void* stream);
+
+/* ---- causal attention with sigmoid weights (no softmax) ---------------------------------------------
+ * out[t, h] = sum over the keys j <= position(t) of t's sequence of sigmoid((q[t, h] . K[j, g]) * scale * temp[h] + bias[h])
+ *   * V[j, g], g = h / (heads / kv_heads); K / V caches [slots, kv_heads, head_dim / v_head_dim] contiguous, reached through
+ *   req_to_token.  `blocks` lists runs (first token, count <= mi355_sigmoid_attention_block_tokens(...)) of consecutive
+ *   tokens of one sequence; null = one token per run and num_blocks = tokens, and then num_splits > 1 cuts every token's
+ *   keys into that many ranges whose partial sums (split_scratch: num_splits * tokens * heads * v_head_dim floats) a second
+ *   launch adds.  The new tokens' keys and values must be in the caches already. */
+int mi355_sigmoid_attention_block_tokens(int heads, int kv_heads, int dtype);
+int mi355_sigmoid_attention(void* out, const void* q, const void* k_cache, const void* v_cache, const int32_t* req_to_token,
+                            const int64_t* req_pool_indices, const int32_t* tok_req, const int64_t* positions,
+                            const int32_t* blocks, int64_t num_blocks, const float* temp, const float* bias,
+                            int64_t q_token_stride, int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride,
+                            int64_t req_to_token_stride, int heads, int kv_heads, int head_dim, int v_head_dim, float scale,
+                            int num_splits, float* split_scratch, int64_t tokens, int dtype, void* stream);
+
+/* ---- mixture of experts ------------------------------------------------------------------------------
+ * mi355_moe_route_grouped: s = sigmoid(logits) (fp32 [tokens, num_experts]); selection on s + correction: experts form
+ *   n_groups equal groups of neighbours, a group scores the sum of its two largest selection scores (its only one, for
+ *   groups of one), the keep_groups best groups stay, the `top` largest selection scores among them are chosen (ties: the
+ *   smaller index); weights[t][k] = s[chosen] / (sum of the chosen s + 1e-20) * scale.
+ * mi355_moe_align: sorts the tokens * top (token, choice) pairs by expert into blocks of mi355_moe_block_rows() rows of
+ *   one expert each: src_row[p] = token of sorted row p or -1 (padding), rows[pair] = p, tile_expert[block] = its expert,
+ *   *n_tiles = blocks in use.  `padded` (a multiple of the block) must be at least pairs + min(experts, pairs) * (block - 1).
+ * mi355_moe_grouped_linear: out[p][.] = act(weight[tile_expert[p / block]] . in[gather ? src_row[p] : p]) for every sorted
+ *   row p of a block in use (0 for padding rows); weight [experts, n, k]; act = erf-GELU when `gelu`. */
+int mi355_moe_route_grouped(int32_t* ids, float* weights, const float* logits, const float* correction, int64_t tokens,
+                            int num_experts, int top, int n_groups, int keep_groups, float scale, void* stream);
+int mi355_moe_block_rows(void);
+int mi355_moe_align(int32_t* src_row, int32_t* rows, int32_t* tile_expert, int32_t* n_tiles, const int32_t* ids, int64_t tokens,
+                    int top, int num_experts, int64_t padded, void* stream);
+int mi355_moe_grouped_linear(void* out, const void* in, int64_t in_stride, const void* weight, const int32_t* src_row,
+                             const int32_t* tile_expert, const int32_t* n_tiles, int gather, int gelu, int64_t padded, int n, int k,
+                             int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -103,6 +103,18 @@ _SIGNATURES = {
     "mi355_gated_residual_add": (I, [P, P, P, P, P, P, P, L, L, L, L, L, I, P]),
     "mi355_latent_norms_rope_write": (I, [P, P, P, P, P, P, P, P, L, L, I, I, I, I, L, F, I, P]),
     "mi355_latent_window_attention_block_tokens": (I, [I, I, I, I]),
+    "mi355_scaled_add_group_rmsnorm": (I, [P, P, P, P, L, P, P, I, F, P, L, L, I, F, I, P]),
+    "mi355_rmsnorm_residual_add": (I, [P, P, P, L, P, L, L, F, I, P]),
+    "mi355_head_norm_rope": (I, [P, P, P, P, P, P, L, I, I, L, L, L, L, L, I, I, F, F, I, I, P]),
+    "mi355_head_rmsnorm_gate": (I, [P, P, P, P, L, L, I, I, F, I, P]),
+    "mi355_gelu_tanh_mul_rows": (I, [P, P, L, P, L, L, L, P, L, L, I, P]),
+    "mi355_linear_recurrence": (I, [P, P, P, P, P, P, P, P, P, P, P, P, P, L, I, I, I, L, L, L, L, F, F, I, I, P]),
+    "mi355_sigmoid_attention_block_tokens": (I, [I, I, I]),
+    "mi355_sigmoid_attention": (I, [P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, I, I, I, I, F, I, P, L, I, P]),
+    "mi355_moe_route_grouped": (I, [P, P, P, P, L, I, I, I, I, F, P]),
+    "mi355_moe_block_rows": (I, []),
+    "mi355_moe_align": (I, [P, P, P, P, P, L, I, I, L, P]),
+    "mi355_moe_grouped_linear": (I, [P, P, L, P, P, P, P, I, I, L, I, I, I, P]),
     "mi355_latent_window_attention": (I, [P, P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, L, L, L, I, I, I, I, I, F, I, P, L, I, P]),
 }
 

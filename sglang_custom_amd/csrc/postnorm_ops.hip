@@ -1,0 +1,285 @@
+// Kernels around a 32-bit residual stream that is normed AFTER every residual sum:
+//   * x <- N(alpha x + branch) * w, N an RMS norm over equal consecutive groups of the row; the branch is a row of a
+//     tensor or a weighted sum of rows picked by an index list (the outputs of a token's experts); the kernel also
+//     writes the activation-dtype copy of the new row,
+//   * x <- x + y / rms(y) * w with the same second output,
+//   * per (token, head): optional RMS norm with a weight shared by the heads, rotation of the leading features by
+//     position-dependent angles in either pairing, a scale; to a tensor or straight into cache rows,
+//   * per (token, head): fp32 row / rms(row) (* weight) * silu(gate) in the activation dtype,
+//   * gelu_tanh(gate) * table[id][column window].
+// Every reduction, normalisation, angle and gate runs in fp32 whatever the activation dtype T is.
+#include "common.cuh"
+
+#include <algorithm>
+
+namespace mi355 {
+namespace {
+
+__device__ __forceinline__ float pn_gelu_tanh(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float pn_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// One workgroup per token.  sm holds the row (D floats) and then one 1/rms per group.
+template <typename T>
+__global__ __launch_bounds__(256) void scaled_add_group_rmsnorm_kernel(
+    float* x_out, T* __restrict__ h_out, const float* x, const T* __restrict__ branch,
+    int64_t branch_stride, const int32_t* __restrict__ rows, const float* __restrict__ coef, int n_branch, float alpha,
+    const T* __restrict__ w, int64_t D, int groups, float eps) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  __shared__ float red[16];
+  float* row = sm;
+  float* inv = sm + D;
+  const int64_t t = blockIdx.x;
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+    float s = alpha * x[t * D + i];
+    if (branch != nullptr) {
+      if (rows == nullptr) {
+        s += to_f32(branch[t * branch_stride + i]);
+      } else {
+        float b = 0.f;
+        for (int j = 0; j < n_branch; ++j)      // fixed order: the sum does not depend on where the rows lie
+          b += coef[t * n_branch + j] * to_f32(branch[(int64_t)rows[t * n_branch + j] * branch_stride + i]);
+        s += b;
+      }
+    }
+    row[i] = s;
+  }
+  __syncthreads();
+  const int64_t gs = D / groups;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  if (groups >= nw) {
+    for (int g = wv; g < groups; g += nw) {
+      float q = 0.f;
+      for (int64_t i = lane; i < gs; i += 64) q += row[g * gs + i] * row[g * gs + i];
+      q = wave_sum(q);
+      if (lane == 0) inv[g] = 1.0f / sqrtf(q / (float)gs + eps);
+    }
+    __syncthreads();
+  } else {
+    for (int g = 0; g < groups; ++g) {
+      float q = 0.f;
+      for (int64_t i = threadIdx.x; i < gs; i += blockDim.x) q += row[g * gs + i] * row[g * gs + i];
+      q = block_sum(q, red);
+      if (threadIdx.x == 0) inv[g] = 1.0f / sqrtf(q / (float)gs + eps);
+    }
+    __syncthreads();
+  }
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+    const float y = row[i] * inv[i / gs] * to_f32(w[i]);
+    if (x_out != nullptr) x_out[t * D + i] = y;
+    if (h_out != nullptr) h_out[t * D + i] = from_f32<T>(y);
+  }
+}
+
+// One workgroup per token: x[t] += y[t] / sqrt(mean(y[t]^2) + eps) * w
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_residual_add_kernel(float* __restrict__ x, T* __restrict__ h_out,
+                                                                   const T* __restrict__ y, int64_t y_stride,
+                                                                   const T* __restrict__ w, int64_t D, float eps) {
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  float q = 0.f;
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+    const float v = to_f32(y[t * y_stride + i]);
+    q += v * v;
+  }
+  q = block_sum(q, red);
+  const float inv = 1.0f / sqrtf(q / (float)D + eps);
+  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+    const float v = x[t * D + i] + to_f32(y[t * y_stride + i]) * inv * to_f32(w[i]);
+    x[t * D + i] = v;
+    if (h_out != nullptr) h_out[t * D + i] = from_f32<T>(v);
+  }
+}
+
+// One wave per (token, head); four per workgroup.  sm: 4 rows of d floats.
+template <typename T, typename OT>
+__global__ __launch_bounds__(256) void head_norm_rope_kernel(
+    OT* __restrict__ out, const T* __restrict__ src, const T* __restrict__ w, const int64_t* __restrict__ positions,
+    const int64_t* __restrict__ loc, const float* __restrict__ inv_freq, int64_t tokens, int heads, int d, int64_t src_token_stride,
+    int64_t src_head_stride, int64_t out_token_stride, int64_t out_head_stride, int rot_dims, int interleaved, float scale,
+    float eps) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t idx = (int64_t)blockIdx.x * 4 + wv;
+  const bool valid = idx < tokens * heads;
+  const int64_t t = valid ? idx / heads : 0;
+  const int h = valid ? (int)(idx - t * heads) : 0;
+  float* row = sm + (int64_t)wv * d;
+  const T* s = src + t * src_token_stride + (int64_t)h * src_head_stride;
+  float q = 0.f;
+  if (valid) {
+    for (int i = lane; i < d; i += 64) {
+      const float v = to_f32(s[i]);
+      row[i] = v;
+      q += v * v;
+    }
+  }
+  float inv = 1.0f;
+  if (w != nullptr) {
+    q = wave_sum(q);
+    inv = 1.0f / sqrtf(q / (float)d + eps);
+  }
+  __syncthreads();
+  if (!valid) return;
+  const float pos = (float)positions[t];
+  const int64_t orow = loc != nullptr ? loc[t] : t;
+  OT* o = out + orow * out_token_stride + (int64_t)h * out_head_stride;
+  const int half = rot_dims / 2;
+  for (int i = lane; i < d; i += 64) {
+    float v = row[i] * inv * (w != nullptr ? to_f32(w[i]) : 1.0f);
+    if (i < rot_dims) {
+      int pair, partner;
+      bool second;
+      if (interleaved) {
+        pair = i >> 1;
+        second = (i & 1) != 0;
+        partner = i ^ 1;
+      } else {
+        second = i >= half;
+        pair = second ? i - half : i;
+        partner = second ? i - half : i + half;
+      }
+      const float u = row[partner] * inv * (w != nullptr ? to_f32(w[partner]) : 1.0f);
+      float sn, cs;
+      sincosf(pos * inv_freq[pair], &sn, &cs);
+      // (a, b) -> (a cos - b sin, b cos + a sin): v is a for the first of the pair, b for the second
+      v = second ? v * cs + u * sn : v * cs - u * sn;
+    }
+    o[i] = from_f32<OT>(v * scale);
+  }
+}
+
+// One wave per (token, head): out = o / rms(o) (* w) * silu(gate)
+template <typename T>
+__global__ __launch_bounds__(256) void head_rmsnorm_gate_kernel(T* __restrict__ out, const float* __restrict__ o,
+                                                                const T* __restrict__ w, const T* __restrict__ gate,
+                                                                int64_t gate_stride, int64_t tokens, int heads, int dv, float eps) {
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t idx = (int64_t)blockIdx.x * 4 + wv;
+  if (idx >= tokens * heads) return;
+  const int64_t t = idx / heads;
+  const int h = (int)(idx - t * heads);
+  const float* r = o + idx * dv;
+  float q = 0.f;
+  for (int i = lane; i < dv; i += 64) q += r[i] * r[i];
+  q = wave_sum(q);
+  const float inv = 1.0f / sqrtf(q / (float)dv + eps);
+  const T* g = gate + t * gate_stride + (int64_t)h * dv;
+  T* dst = out + idx * dv;
+  for (int i = lane; i < dv; i += 64) {
+    const float z = to_f32(g[i]);
+    const float n = r[i] * inv * (w != nullptr ? to_f32(w[i]) : 1.0f);
+    dst[i] = from_f32<T>(n * z * pn_sigmoid(z));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_tanh_mul_rows_kernel(T* __restrict__ out, const T* __restrict__ gate,
+                                                                 int64_t gate_stride, const T* __restrict__ table,
+                                                                 int64_t table_stride, int64_t col_off,
+                                                                 const int64_t* __restrict__ ids, int64_t rows, int64_t d) {
+  const int64_t n = rows * d;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = idx / d, i = idx - r * d;
+    out[idx] = from_f32<T>(pn_gelu_tanh(to_f32(gate[r * gate_stride + i])) * to_f32(table[ids[r] * table_stride + col_off + i]));
+  }
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+int mi355_scaled_add_group_rmsnorm(float* x_out, void* h_out, const float* x, const void* branch, int64_t branch_stride,
+                                   const int32_t* rows, const float* coef, int n_branch, float alpha, const void* weight,
+                                   int64_t tokens, int64_t hidden, int groups, float eps, int dtype, void* stream) {
+  MI355_REQUIRE(x && weight && (x_out || h_out), MI355_ERR_INVALID, "scaled_add_group_rmsnorm: null pointer");
+  MI355_REQUIRE(tokens >= 0 && hidden > 0 && groups > 0 && hidden % groups == 0 && groups <= 4096 && hidden <= 32768,
+                MI355_ERR_INVALID, "scaled_add_group_rmsnorm: bad shape");
+  MI355_REQUIRE((rows == nullptr) == (coef == nullptr) && (rows == nullptr || (branch && n_branch > 0)), MI355_ERR_INVALID,
+                "scaled_add_group_rmsnorm: rows, coef and the branch come together");
+  if (tokens == 0) return MI355_OK;
+  const size_t lds = (size_t)(hidden + groups) * sizeof(float);
+  MI355_DISPATCH_DTYPE(dtype, "scaled_add_group_rmsnorm", {
+    hipLaunchKernelGGL((scaled_add_group_rmsnorm_kernel<T>), dim3((unsigned)tokens), dim3(256), lds, (hipStream_t)stream, x_out,
+                       (T*)h_out, x, (const T*)branch, branch_stride, rows, coef, n_branch, alpha, (const T*)weight, hidden,
+                       groups, eps);
+  });
+  MI355_CHECK_LAUNCH("scaled_add_group_rmsnorm");
+  return MI355_OK;
+}
+
+int mi355_rmsnorm_residual_add(float* x, void* h_out, const void* y, int64_t y_stride, const void* weight, int64_t tokens,
+                               int64_t hidden, float eps, int dtype, void* stream) {
+  MI355_REQUIRE(x && y && weight, MI355_ERR_INVALID, "rmsnorm_residual_add: null pointer");
+  MI355_REQUIRE(tokens >= 0 && hidden > 0 && y_stride >= hidden, MI355_ERR_INVALID, "rmsnorm_residual_add: bad shape");
+  if (tokens == 0) return MI355_OK;
+  MI355_DISPATCH_DTYPE(dtype, "rmsnorm_residual_add", {
+    hipLaunchKernelGGL((rmsnorm_residual_add_kernel<T>), dim3((unsigned)tokens), dim3(256), 0, (hipStream_t)stream, x, (T*)h_out,
+                       (const T*)y, y_stride, (const T*)weight, hidden, eps);
+  });
+  MI355_CHECK_LAUNCH("rmsnorm_residual_add");
+  return MI355_OK;
+}
+
+int mi355_head_norm_rope(void* out, const void* src, const void* weight, const int64_t* positions, const int64_t* loc,
+                         const float* inv_freq, int64_t tokens, int heads, int head_dim, int64_t src_token_stride,
+                         int64_t src_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t out_rows, int rot_dims,
+                         int interleaved, float scale, float eps, int dtype, int out_dtype, void* stream) {
+  MI355_REQUIRE(out && src && positions, MI355_ERR_INVALID, "head_norm_rope: null pointer");
+  MI355_REQUIRE(tokens >= 0 && heads > 0 && head_dim > 0 && head_dim <= 4096 && out_rows >= 0, MI355_ERR_INVALID,
+                "head_norm_rope: bad shape");
+  MI355_REQUIRE(rot_dims >= 0 && rot_dims <= head_dim && rot_dims % 2 == 0 && (rot_dims == 0 || inv_freq), MI355_ERR_INVALID,
+                "head_norm_rope: rot_dims must be even, at most head_dim, and come with frequencies");
+  MI355_REQUIRE(out_dtype == dtype || out_dtype == MI355_F32, MI355_ERR_UNSUPPORTED,
+                "head_norm_rope: the result is written in the input's type or in fp32");
+  if (tokens == 0) return MI355_OK;
+  const size_t lds = (size_t)4 * head_dim * sizeof(float);
+  const unsigned grid = (unsigned)((tokens * heads + 3) / 4);
+  MI355_DISPATCH_DTYPE(dtype, "head_norm_rope", {
+    if (out_dtype == dtype) {
+      hipLaunchKernelGGL((head_norm_rope_kernel<T, T>), dim3(grid), dim3(256), lds, (hipStream_t)stream, (T*)out, (const T*)src,
+                         (const T*)weight, positions, loc, inv_freq, tokens, heads, head_dim, src_token_stride, src_head_stride,
+                         out_token_stride, out_head_stride, rot_dims, interleaved, scale, eps);
+    } else {
+      hipLaunchKernelGGL((head_norm_rope_kernel<T, float>), dim3(grid), dim3(256), lds, (hipStream_t)stream, (float*)out,
+                         (const T*)src, (const T*)weight, positions, loc, inv_freq, tokens, heads, head_dim, src_token_stride,
+                         src_head_stride, out_token_stride, out_head_stride, rot_dims, interleaved, scale, eps);
+    }
+  });
+  MI355_CHECK_LAUNCH("head_norm_rope");
+  return MI355_OK;
+}
+
+int mi355_head_rmsnorm_gate(void* out, const float* o, const void* weight, const void* gate, int64_t gate_stride, int64_t tokens,
+                            int heads, int value_dim, float eps, int dtype, void* stream) {
+  MI355_REQUIRE(out && o && gate, MI355_ERR_INVALID, "head_rmsnorm_gate: null pointer");
+  MI355_REQUIRE(tokens >= 0 && heads > 0 && value_dim > 0 && gate_stride >= (int64_t)heads * value_dim, MI355_ERR_INVALID,
+                "head_rmsnorm_gate: bad shape");
+  if (tokens == 0) return MI355_OK;
+  const unsigned grid = (unsigned)((tokens * heads + 3) / 4);
+  MI355_DISPATCH_DTYPE(dtype, "head_rmsnorm_gate", {
+    hipLaunchKernelGGL((head_rmsnorm_gate_kernel<T>), dim3(grid), dim3(256), 0, (hipStream_t)stream, (T*)out, o, (const T*)weight,
+                       (const T*)gate, gate_stride, tokens, heads, value_dim, eps);
+  });
+  MI355_CHECK_LAUNCH("head_rmsnorm_gate");
+  return MI355_OK;
+}
+
+int mi355_gelu_tanh_mul_rows(void* out, const void* gate, int64_t gate_stride, const void* table, int64_t table_rows,
+                             int64_t table_stride, int64_t col_off, const int64_t* ids, int64_t rows, int64_t d, int dtype,
+                             void* stream) {
+  MI355_REQUIRE(out && gate && table && ids, MI355_ERR_INVALID, "gelu_tanh_mul_rows: null pointer");
+  MI355_REQUIRE(rows >= 0 && d > 0 && gate_stride >= d && col_off >= 0 && col_off + d <= table_stride && table_rows > 0,
+                MI355_ERR_INVALID, "gelu_tanh_mul_rows: bad shape");
+  if (rows == 0) return MI355_OK;
+  const int grid = (int)std::min<int64_t>((rows * d + 255) / 256, 256 * 16);
+  MI355_DISPATCH_DTYPE(dtype, "gelu_tanh_mul_rows", {
+    hipLaunchKernelGGL((gelu_tanh_mul_rows_kernel<T>), dim3(grid), dim3(256), 0, (hipStream_t)stream, (T*)out, (const T*)gate,
+                       gate_stride, (const T*)table, table_stride, col_off, ids, rows, d);
+  });
+  MI355_CHECK_LAUNCH("gelu_tanh_mul_rows");
+  return MI355_OK;
+}

@@ -1,0 +1,169 @@
+// Linear recurrence with one fp32 matrix per (sequence, head):
+//     S_t = diag(a_t) S_{t-1} + k_t v_t^T        S [dk, dv]
+//     o_t = S_t^T (q_t * q_scale)
+// a_t either per key channel and token, a = exp(logsigmoid(z + b) / tau) from gate logits z (fp32), or one number per head.
+//
+// One workgroup per (sequence of the step, head, block of 32 value columns): it loads the block's dk x 32 part of the
+// sequence's matrix (zero at position 0), runs the step's tokens of that sequence through it in order, and stores it
+// back.  A lane owns ONE column and R consecutive key channels of it in registers (8 lanes share a column, a wave holds 8
+// columns, the 4 waves 32); per token it does R (mul, fma, fma) and the 8 partial dot products of a column meet over
+// three lane exchanges.  q, k and the decays of the next TC tokens are staged in LDS (all fp32 from there on).  A decode
+// step is the same launch with one token per sequence; what bounds it then is the matrix's trip through HBM, which each
+// workgroup makes in whole 128-byte rows.
+#include "common.cuh"
+
+namespace mi355 {
+namespace {
+
+constexpr int RC_COLS = 32;   // value columns per workgroup
+constexpr int RC_RG = 8;      // lanes that share a column
+constexpr int RC_TC = 16;     // tokens staged at a time
+
+__device__ __forceinline__ float log_sigmoid_f(float z) {
+  // log(1 / (1 + exp(-z))) without overflow on either side
+  return fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+}
+
+template <typename QT, typename VT, int R>
+__global__ __launch_bounds__(256) void linear_recurrence_kernel(
+    float* __restrict__ out, float* __restrict__ state, const QT* __restrict__ q, const QT* __restrict__ k,
+    const VT* __restrict__ v, const float* __restrict__ gate_logits, const VT* __restrict__ gate_bias,
+    const float* __restrict__ head_decay, const int32_t* __restrict__ req_to_state, const int64_t* __restrict__ req_pool_indices,
+    const int32_t* __restrict__ seg_start, const int32_t* __restrict__ seg_len, const int64_t* __restrict__ positions, int heads,
+    int dk, int dv, int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride, int64_t gate_token_stride,
+    float q_scale, float inv_tau) {
+  constexpr int DKP = R * RC_RG;     // key channels with padding
+  __shared__ __attribute__((aligned(16))) float qs[RC_TC][DKP];
+  __shared__ __attribute__((aligned(16))) float ks[RC_TC][DKP];
+  __shared__ __attribute__((aligned(16))) float as[RC_TC][DKP];
+  __shared__ float vs[RC_TC][RC_COLS];
+  const int b = blockIdx.z, h = blockIdx.y, c0 = blockIdx.x * RC_COLS;
+  const int tid = threadIdx.x;
+  const int rg = tid & (RC_RG - 1), cl = tid >> 3;       // lane = column * 8 + row group
+  const int col = c0 + cl;
+  const int64_t t0 = seg_start != nullptr ? seg_start[b] : b;
+  const int n = seg_len != nullptr ? seg_len[b] : 1;
+  if (n <= 0) return;
+  const int64_t slot = req_to_state[req_pool_indices[b]];
+  float* sp = state + ((slot * heads + h) * (int64_t)dk) * dv;
+  float S[R];
+  const bool fresh = positions[t0] == 0;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int i = rg * R + r;
+    S[r] = (!fresh && i < dk && col < dv) ? sp[(int64_t)i * dv + col] : 0.f;
+  }
+  const float hd = head_decay != nullptr ? head_decay[h] : 1.f;
+  for (int base = 0; base < n; base += RC_TC) {
+    const int m = min(RC_TC, n - base);
+    __syncthreads();
+    for (int e = tid; e < m * DKP; e += 256) {
+      const int tt = e / DKP, i = e - tt * DKP;
+      const int64_t t = t0 + base + tt;
+      float qv = 0.f, kv = 0.f, av = 1.f;
+      if (i < dk) {
+        qv = to_f32(q[t * q_token_stride + (int64_t)h * dk + i]) * q_scale;
+        kv = to_f32(k[t * k_token_stride + (int64_t)h * dk + i]);
+        if (gate_logits != nullptr) {
+          float z = gate_logits[t * gate_token_stride + (int64_t)h * dk + i];
+          if (gate_bias != nullptr) z += to_f32(gate_bias[(int64_t)h * dk + i]);
+          av = expf(log_sigmoid_f(z) * inv_tau);
+        } else {
+          av = hd;
+        }
+      }
+      qs[tt][i] = qv;
+      ks[tt][i] = kv;
+      as[tt][i] = av;
+    }
+    for (int e = tid; e < m * RC_COLS; e += 256) {
+      const int tt = e / RC_COLS, c = e - tt * RC_COLS;
+      vs[tt][c] = (c0 + c < dv) ? to_f32(v[(t0 + base + tt) * v_token_stride + (int64_t)h * dv + c0 + c]) : 0.f;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < m; ++tt) {
+      const float vj = vs[tt][cl];
+      float acc = 0.f;
+#pragma unroll
+      for (int r4 = 0; r4 < R; r4 += 4) {
+        const float4 a4 = *reinterpret_cast<const float4*>(&as[tt][rg * R + r4]);
+        const float4 k4 = *reinterpret_cast<const float4*>(&ks[tt][rg * R + r4]);
+        const float4 q4 = *reinterpret_cast<const float4*>(&qs[tt][rg * R + r4]);
+        S[r4 + 0] = fmaf(a4.x, S[r4 + 0], k4.x * vj);
+        S[r4 + 1] = fmaf(a4.y, S[r4 + 1], k4.y * vj);
+        S[r4 + 2] = fmaf(a4.z, S[r4 + 2], k4.z * vj);
+        S[r4 + 3] = fmaf(a4.w, S[r4 + 3], k4.w * vj);
+        acc = fmaf(S[r4 + 0], q4.x, acc);
+        acc = fmaf(S[r4 + 1], q4.y, acc);
+        acc = fmaf(S[r4 + 2], q4.z, acc);
+        acc = fmaf(S[r4 + 3], q4.w, acc);
+      }
+      acc += __shfl_xor(acc, 1, 64);
+      acc += __shfl_xor(acc, 2, 64);
+      acc += __shfl_xor(acc, 4, 64);
+      if (rg == 0 && col < dv) out[((t0 + base + tt) * heads + h) * (int64_t)dv + col] = acc;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int i = rg * R + r;
+    if (i < dk && col < dv) sp[(int64_t)i * dv + col] = S[r];
+  }
+}
+
+template <typename QT, typename VT>
+int launch_recurrence(float* out, float* state, const void* q, const void* k, const void* v, const float* gate_logits,
+                      const void* gate_bias, const float* head_decay, const int32_t* req_to_state, const int64_t* req_pool_indices,
+                      const int32_t* seg_start, const int32_t* seg_len, const int64_t* positions, int64_t batch, int heads, int dk,
+                      int dv, int64_t qs, int64_t ks, int64_t vs, int64_t gs, float q_scale, float tau, hipStream_t stream) {
+  const dim3 grid((unsigned)cdiv(dv, RC_COLS), (unsigned)heads, (unsigned)batch);
+#define MI355_RC_LAUNCH(R)                                                                                                     \
+  hipLaunchKernelGGL((linear_recurrence_kernel<QT, VT, R>), grid, dim3(256), 0, stream, out, state, (const QT*)q, (const QT*)k, \
+                     (const VT*)v, gate_logits, (const VT*)gate_bias, head_decay, req_to_state, req_pool_indices, seg_start,   \
+                     seg_len, positions, heads, dk, dv, qs, ks, vs, gs, q_scale, 1.0f / tau)
+  if (dk <= 32) MI355_RC_LAUNCH(4);
+  else if (dk <= 64) MI355_RC_LAUNCH(8);
+  else if (dk <= 128) MI355_RC_LAUNCH(16);
+  else MI355_RC_LAUNCH(32);
+#undef MI355_RC_LAUNCH
+  return MI355_OK;
+}
+
+}  // namespace
+}  // namespace mi355
+
+using namespace mi355;
+
+int mi355_linear_recurrence(float* out, float* state, const void* q, const void* k, const void* v, const float* gate_logits,
+                            const void* gate_bias, const float* head_decay, const int32_t* req_to_state,
+                            const int64_t* req_pool_indices, const int32_t* seg_start, const int32_t* seg_len,
+                            const int64_t* positions, int64_t batch, int heads, int key_dim, int value_dim, int64_t q_token_stride,
+                            int64_t k_token_stride, int64_t v_token_stride, int64_t gate_token_stride, float q_scale, float tau,
+                            int qk_dtype, int v_dtype, void* stream) {
+  MI355_REQUIRE(out && state && q && k && v && req_to_state && req_pool_indices && positions, MI355_ERR_INVALID,
+                "linear_recurrence: null pointer");
+  MI355_REQUIRE((gate_logits != nullptr) != (head_decay != nullptr), MI355_ERR_INVALID,
+                "linear_recurrence: the decay is either gate logits per channel or one number per head");
+  MI355_REQUIRE((seg_start == nullptr) == (seg_len == nullptr), MI355_ERR_INVALID,
+                "linear_recurrence: seg_start and seg_len come together");
+  MI355_REQUIRE(batch >= 0 && batch <= 65535 && heads > 0 && heads <= 65535 && key_dim > 0 && value_dim > 0 && tau > 0.f,
+                MI355_ERR_INVALID, "linear_recurrence: bad shape");
+  MI355_REQUIRE(key_dim <= 256, MI355_ERR_UNSUPPORTED, "linear_recurrence: key width %d above 256", key_dim);
+  MI355_REQUIRE(qk_dtype == v_dtype || qk_dtype == MI355_F32, MI355_ERR_UNSUPPORTED,
+                "linear_recurrence: q and k come in the type of v or in fp32");
+  if (batch == 0) return MI355_OK;
+  int rc = MI355_OK;
+  MI355_DISPATCH_DTYPE(v_dtype, "linear_recurrence", {
+    if (qk_dtype == v_dtype)
+      rc = launch_recurrence<T, T>(out, state, q, k, v, gate_logits, gate_bias, head_decay, req_to_state, req_pool_indices,
+                                   seg_start, seg_len, positions, batch, heads, key_dim, value_dim, q_token_stride, k_token_stride,
+                                   v_token_stride, gate_token_stride, q_scale, tau, (hipStream_t)stream);
+    else
+      rc = launch_recurrence<float, T>(out, state, q, k, v, gate_logits, gate_bias, head_decay, req_to_state, req_pool_indices,
+                                       seg_start, seg_len, positions, batch, heads, key_dim, value_dim, q_token_stride,
+                                       k_token_stride, v_token_stride, gate_token_stride, q_scale, tau, (hipStream_t)stream);
+  });
+  if (rc != MI355_OK) return rc;
+  MI355_CHECK_LAUNCH("linear_recurrence");
+  return MI355_OK;
+}

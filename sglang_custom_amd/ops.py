@@ -1254,3 +1254,219 @@ def latent_window_attention(qa: torch.Tensor, qr: torch.Tensor, cache: torch.Ten
         gate.stride(0) if gate is not None else 0, req_to_token.stride(0), H, rank, rope_dim, rot_dims, int(window), float(scale),
         int(num_splits), _p(scratch), T, _dt(qa), _stream(qa)), "latent_window_attention")
     return out
+
+
+# ------------------------------------------------------- post-norm fp32 stream, head norms and rotations
+def scaled_add_group_rmsnorm(x: torch.Tensor, branch: Optional[torch.Tensor], alpha: float, weight: torch.Tensor, groups: int,
+                             eps: float, rows: Optional[torch.Tensor] = None, coef: Optional[torch.Tensor] = None,
+                             inplace: bool = True) -> torch.Tensor:
+    """y = N(alpha * x + branch) * weight, N the RMS norm over `groups` equal parts of the row.  inplace: x <- y; returns y
+    in the weight's dtype (x itself for an fp32 model).  rows int32 [T, n] / coef fp32 [T, n]: token t's branch is
+    sum_j coef[t, j] * branch[rows[t, j]]."""
+    _gpu(x, branch, weight, rows, coef)
+    assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and weight.is_contiguous() and weight.numel() == x.shape[1]
+    T, D = x.shape
+    n_branch = 1
+    if rows is not None:
+        assert rows.dtype == torch.int32 and coef.dtype == torch.float32 and rows.shape == coef.shape and rows.shape[0] == T
+        assert rows.is_contiguous() and coef.is_contiguous() and branch is not None
+        n_branch = rows.shape[1]
+    if branch is not None:
+        assert branch.dim() == 2 and branch.shape[1] == D and branch.stride(1) == 1 and branch.dtype == weight.dtype
+        assert rows is not None or branch.shape[0] == T
+    same = weight.dtype == torch.float32
+    h = None if (same and inplace) else torch.empty((T, D), dtype=weight.dtype, device=x.device)
+    check(_lib_().mi355_scaled_add_group_rmsnorm(x.data_ptr() if inplace else None, _p(h), x.data_ptr(), _p(branch),
+                                                 branch.stride(0) if branch is not None else 0, _p(rows), _p(coef), n_branch,
+                                                 float(alpha), weight.data_ptr(), T, D, int(groups), float(eps), _dt(weight),
+                                                 _stream(x)), "scaled_add_group_rmsnorm")
+    return x if h is None else h
+
+
+def rmsnorm_residual_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """x += y / sqrt(mean(y^2) + eps) * weight in place on the fp32 rows; returns the new x in the weight's dtype."""
+    _gpu(x, y, weight)
+    assert x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and y.shape == x.shape and y.stride(1) == 1
+    assert y.dtype == weight.dtype and weight.is_contiguous() and weight.numel() == x.shape[1]
+    T, D = x.shape
+    h = None if weight.dtype == torch.float32 else torch.empty((T, D), dtype=weight.dtype, device=x.device)
+    check(_lib_().mi355_rmsnorm_residual_add(x.data_ptr(), _p(h), y.data_ptr(), y.stride(0), weight.data_ptr(), T, D, float(eps),
+                                             _dt(weight), _stream(x)), "rmsnorm_residual_add")
+    return x if h is None else h
+
+
+def head_norm_rope(src: torch.Tensor, weight: Optional[torch.Tensor], eps: float, positions: torch.Tensor, inv_freq: torch.Tensor,
+                   rot_dims: int, interleaved: bool, scale: float, out_dtype: torch.dtype, cache: Optional[torch.Tensor] = None,
+                   loc: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """src [T, H, d] (token / head strides free) -> optional RMS norm per head, rotation of the first rot_dims features,
+    scale; to a new [T, H, d] tensor of out_dtype, or into cache[loc[t]] ([slots, H, d]) when a cache is given."""
+    _gpu(src, weight, positions, inv_freq, cache, loc)
+    T, H, d = src.shape
+    assert src.stride(2) == 1 and positions.dtype == torch.int64 and positions.is_contiguous()
+    assert weight is None or (weight.dtype == src.dtype and weight.numel() == d and weight.is_contiguous())
+    assert rot_dims == 0 or (inv_freq.dtype == torch.float32 and inv_freq.numel() >= rot_dims // 2)
+    if cache is not None:
+        assert cache.is_contiguous() and cache.shape[1:] == (H, d) and loc is not None and loc.dtype == torch.int64
+        assert loc.is_contiguous() and loc.numel() == T
+        out, out_dtype = cache, cache.dtype
+    else:
+        out = torch.empty((T, H, d), dtype=out_dtype, device=src.device)
+        loc = None
+    check(_lib_().mi355_head_norm_rope(out.data_ptr(), src.data_ptr(), _p(weight), positions.data_ptr(), _p(loc),
+                                       _p(inv_freq) if rot_dims else None, T, H, d, src.stride(0), src.stride(1), out.stride(0),
+                                       out.stride(1), out.shape[0], int(rot_dims), int(bool(interleaved)), float(scale),
+                                       float(eps), _dt(src), _DT[out_dtype], _stream(src)), "head_norm_rope")
+    return out
+
+
+def head_rmsnorm_gate(o: torch.Tensor, weight: Optional[torch.Tensor], gate: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """o fp32 [T, H, dv] -> o / rms(o) (* weight) * silu(gate) as [T, H * dv] of the gate's dtype; gate [T, H * dv] row-strided."""
+    _gpu(o, weight, gate)
+    T, H, dv = o.shape
+    assert o.dtype == torch.float32 and o.is_contiguous() and gate.shape == (T, H * dv) and gate.stride(1) == 1
+    assert gate.dtype == out_dtype and (weight is None or (weight.dtype == out_dtype and weight.numel() == dv and weight.is_contiguous()))
+    out = torch.empty((T, H * dv), dtype=out_dtype, device=o.device)
+    check(_lib_().mi355_head_rmsnorm_gate(out.data_ptr(), o.data_ptr(), _p(weight), gate.data_ptr(), gate.stride(0), T, H, dv,
+                                          float(eps), _dt(gate), _stream(o)), "head_rmsnorm_gate")
+    return out
+
+
+def gelu_tanh_mul_rows(gate: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col_off: int) -> torch.Tensor:
+    """gelu_tanh(gate [T, d]) * table[ids, col_off: col_off + d]."""
+    _gpu(gate, table, ids)
+    T, d = gate.shape
+    assert gate.stride(1) == 1 and table.dim() == 2 and table.stride(1) == 1 and table.dtype == gate.dtype
+    assert ids.dtype == torch.int64 and ids.is_contiguous() and ids.numel() == T and 0 <= col_off and col_off + d <= table.shape[1]
+    out = torch.empty((T, d), dtype=gate.dtype, device=gate.device)
+    check(_lib_().mi355_gelu_tanh_mul_rows(out.data_ptr(), gate.data_ptr(), gate.stride(0), table.data_ptr(), table.shape[0],
+                                           table.stride(0), int(col_off), ids.data_ptr(), T, d, _dt(gate), _stream(gate)),
+          "gelu_tanh_mul_rows")
+    return out
+
+
+# ------------------------------------------------------- linear recurrence over per-sequence matrices
+def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, state: torch.Tensor,
+                      req_to_state: torch.Tensor, req_pool_indices: torch.Tensor, positions: torch.Tensor, q_scale: float,
+                      gate_logits: Optional[torch.Tensor] = None, gate_bias: Optional[torch.Tensor] = None, tau: float = 1.0,
+                      head_decay: Optional[torch.Tensor] = None, tok_req=None, seg_start=None, seg_len=None) -> torch.Tensor:
+    """S = diag(a) S + k v^T, out = S^T (q * q_scale) per head over every sequence's tokens of the step, on
+    state[slot] ([slots, H, dk, dv] fp32, read unless the sequence starts at position 0, written back).  q, k [T, H, dk]
+    (fp32 or v's dtype), v [T, H, dv]; the decay from gate_logits fp32 [T, H * dk] (+ gate_bias, / tau) or head_decay fp32 [H]."""
+    _gpu(q, k, v, out, state, req_to_state, req_pool_indices, positions, gate_logits, gate_bias, head_decay)
+    T, H, dk = q.shape
+    dv = v.shape[2]
+    assert k.shape == q.shape and v.shape[:2] == (T, H) and q.dtype == k.dtype and q.dtype in (v.dtype, torch.float32)
+    for t in (q, k, v):
+        assert t.stride(2) == 1 and t.stride(1) == t.shape[2], "heads lie side by side in a token's row"
+    assert out.dtype == torch.float32 and out.shape == (T, H, dv) and out.is_contiguous()
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, dk, dv)
+    assert req_to_state.dtype == torch.int32 and req_pool_indices.dtype == torch.int64 and positions.dtype == torch.int64
+    assert (gate_logits is None) != (head_decay is None)
+    if gate_logits is not None:
+        assert gate_logits.dtype == torch.float32 and gate_logits.shape == (T, H * dk) and gate_logits.stride(1) == 1
+        assert gate_bias is None or (gate_bias.dtype == v.dtype and gate_bias.numel() == H * dk and gate_bias.is_contiguous())
+    else:
+        assert head_decay.dtype == torch.float32 and head_decay.numel() == H and head_decay.is_contiguous()
+    _, ss, sl = _seg(tok_req, seg_start, seg_len)
+    B = req_pool_indices.numel()
+    assert seg_start is not None or B == T, "without segments every token is a sequence of its own"
+    check(_lib_().mi355_linear_recurrence(out.data_ptr(), state.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                          _p(gate_logits), _p(gate_bias), _p(head_decay), req_to_state.data_ptr(),
+                                          req_pool_indices.data_ptr(), ss, sl, positions.data_ptr(), B, H, dk, dv, q.stride(0),
+                                          k.stride(0), v.stride(0), gate_logits.stride(0) if gate_logits is not None else 0,
+                                          float(q_scale), float(tau), _dt(q), _dt(v), _stream(q)), "linear_recurrence")
+    return out
+
+
+# ------------------------------------------------------- causal attention with sigmoid weights
+def sigmoid_attention_block_tokens(heads: int, kv_heads: int, dtype: torch.dtype) -> int:
+    """Most consecutive tokens of one sequence that a workgroup of sigmoid_attention takes."""
+    return int(_lib_().mi355_sigmoid_attention_block_tokens(heads, kv_heads, _DT[dtype]))
+
+
+def sigmoid_attention_splits(tokens: int, heads: int, kv_heads: int, max_len: int, dtype: torch.dtype) -> int:
+    """Key ranges per token for a decode-sized launch: enough workgroups to cover the chip twice, at least 128 keys each."""
+    wgs = max(1, tokens * kv_heads * ((heads // kv_heads + 15) // 16))
+    return int(max(1, min(64, (512 + wgs - 1) // wgs, max_len // 128)))
+
+
+def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, req_to_token: torch.Tensor,
+                      req_pool_indices: torch.Tensor, positions: torch.Tensor, temp: torch.Tensor, bias: torch.Tensor, scale: float,
+                      tok_req=None, blocks=None, num_splits: int = 1) -> torch.Tensor:
+    """q [T, H, d], caches [slots, G, d] / [slots, G, dv], out [T, H, dv]; temp / bias fp32 [H]; blocks int32 [n, 2] runs of
+    consecutive tokens of one sequence or None (one token per run)."""
+    _gpu(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, temp, bias, tok_req, blocks)
+    T, H, d = q.shape
+    G, dv = k_cache.shape[1], v_cache.shape[2]
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.shape[2] == d and v_cache.shape[1] == G
+    assert out.shape == (T, H, dv) and q.stride(2) == 1 and out.stride(2) == 1 and q.dtype == out.dtype == k_cache.dtype == v_cache.dtype
+    assert temp.dtype == torch.float32 and bias.dtype == torch.float32 and temp.numel() == H and bias.numel() == H
+    assert temp.is_contiguous() and bias.is_contiguous()
+    assert req_to_token.dtype == torch.int32 and req_pool_indices.dtype == torch.int64 and positions.dtype == torch.int64
+    assert tok_req is None or (tok_req.dtype == torch.int32 and tok_req.numel() == T)
+    if blocks is not None:
+        assert blocks.dtype == torch.int32 and blocks.dim() == 2 and blocks.shape[1] == 2 and blocks.is_contiguous()
+        nb, num_splits = blocks.shape[0], 1
+    else:
+        nb = T
+    scratch = torch.empty(num_splits * T * H * dv, dtype=torch.float32, device=q.device) if num_splits > 1 else None
+    check(_lib_().mi355_sigmoid_attention(
+        out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), req_to_token.data_ptr(), req_pool_indices.data_ptr(),
+        _p(tok_req), positions.data_ptr(), _p(blocks), nb, temp.data_ptr(), bias.data_ptr(), q.stride(0), q.stride(1),
+        out.stride(0), out.stride(1), req_to_token.stride(0), H, G, d, dv, float(scale), int(num_splits), _p(scratch), T, _dt(q),
+        _stream(q)), "sigmoid_attention")
+    return out
+
+
+# ------------------------------------------------------- mixture of experts
+def moe_route_grouped(logits: torch.Tensor, correction: torch.Tensor, top: int, n_groups: int, keep_groups: int,
+                      scale: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp32 logits [T, E] -> (expert ids int32 [T, top], weights fp32 [T, top])."""
+    _gpu(logits, correction)
+    T, E = logits.shape
+    assert logits.dtype == torch.float32 and logits.is_contiguous() and correction.dtype == torch.float32 and correction.numel() == E
+    ids = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    check(_lib_().mi355_moe_route_grouped(ids.data_ptr(), w.data_ptr(), logits.data_ptr(), correction.data_ptr(), T, E, int(top),
+                                          int(n_groups), int(keep_groups), float(scale), _stream(logits)), "moe_route_grouped")
+    return ids, w
+
+
+class MoePlan:
+    """The sorted layout of a step's (token, expert) pairs, all on the device: src_row int32 [padded] (token of a sorted
+    row, -1 for padding), rows int32 [T, top] (sorted row of a pair), tile_expert int32 [padded / block], n_tiles int32 [1]."""
+    __slots__ = ("src_row", "rows", "tile_expert", "n_tiles", "block", "padded")
+
+    def __init__(self, src_row, rows, tile_expert, n_tiles, block, padded):
+        self.src_row, self.rows, self.tile_expert, self.n_tiles, self.block, self.padded = src_row, rows, tile_expert, n_tiles, block, padded
+
+
+def moe_align(expert_ids: torch.Tensor, num_experts: int) -> MoePlan:
+    _gpu(expert_ids)
+    T, top = expert_ids.shape
+    assert expert_ids.dtype == torch.int32 and expert_ids.is_contiguous()
+    block = int(_lib_().mi355_moe_block_rows())
+    pairs = T * top
+    padded = (pairs + min(num_experts, pairs) * (block - 1) + block - 1) // block * block
+    dev = expert_ids.device
+    src_row = torch.empty(max(padded, 1), dtype=torch.int32, device=dev)
+    rows = torch.empty((T, top), dtype=torch.int32, device=dev)
+    tile_expert = torch.empty(max(padded // block, 1), dtype=torch.int32, device=dev)
+    n_tiles = torch.empty(1, dtype=torch.int32, device=dev)
+    check(_lib_().mi355_moe_align(src_row.data_ptr(), rows.data_ptr(), tile_expert.data_ptr(), n_tiles.data_ptr(),
+                                  expert_ids.data_ptr(), T, top, int(num_experts), padded, _stream(expert_ids)), "moe_align")
+    return MoePlan(src_row, rows, tile_expert, n_tiles, block, padded)
+
+
+def moe_grouped_linear(x: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: bool, gelu: bool) -> torch.Tensor:
+    """out [padded, N] = act(w[expert of the row's block] . x[src_row or the row itself]); rows of blocks not in use are
+    left unwritten (nothing reads them)."""
+    _gpu(x, w)
+    E, N, K = w.shape
+    assert w.is_contiguous() and x.dim() == 2 and x.shape[1] == K and x.stride(1) == 1 and x.dtype == w.dtype
+    assert gather or x.shape[0] == plan.padded
+    out = torch.empty((plan.padded, N), dtype=x.dtype, device=x.device)
+    check(_lib_().mi355_moe_grouped_linear(out.data_ptr(), x.data_ptr(), x.stride(0), w.data_ptr(), plan.src_row.data_ptr(),
+                                           plan.tile_expert.data_ptr(), plan.n_tiles.data_ptr(), int(gather), int(gelu),
+                                           plan.padded, N, K, _dt(x), _stream(x)), "moe_grouped_linear")
+    return out
