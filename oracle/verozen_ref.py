@@ -68,62 +68,78 @@ def rotate_pairs(x: torch.Tensor, dims: int, base: float, neighbours: bool) -> t
 
 
 # ----------------------------------------------------------------------------------- mixers
+def decayed_sum_per_channel(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, log_a: torch.Tensor) -> torch.Tensor:
+    """The recurrence S_t = diag(a_t) S_{t-1} + k_t v_t^T, o_t = S_t^T q_t written as the explicit double sum
+    o_t = sum_{s <= t} (sum_i q_t[i] k_s[i] prod_{s < r <= t} a_r[i]) v_s.   q, k, log_a [T, H, d], v [T, H, dv]."""
+    T, H, _ = q.shape
+    cum = log_a.cumsum(0)                                                     # log of the decay from the start to t
+    o = torch.zeros(T, H, v.shape[-1], dtype=q.dtype)
+    for t in range(T):
+        wgt = torch.exp(cum[t][None] - cum[: t + 1])                          # [s, H, d]: prod_{s < r <= t} a_r
+        score = (q[t][None] * k[: t + 1] * wgt).sum(-1)                       # [s, H]
+        o[t] = torch.einsum("sh,shv->hv", score, v[: t + 1])
+    return o
+
+
+def decayed_sum_per_head(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay) -> torch.Tensor:
+    """o_t = sum_{s <= t} g_h^(t - s) (q_t . k_s) v_s: the same recurrence with one fixed decay per head."""
+    T, H, _ = q.shape
+    t = torch.arange(T, dtype=q.dtype)
+    dist = t[:, None] - t[None, :]
+    o = torch.zeros(T, H, v.shape[-1], dtype=q.dtype)
+    for hd in range(H):
+        g = torch.tensor(float(decay[hd]), dtype=q.dtype)
+        mask = torch.where(dist >= 0, g ** dist.clamp_min(0), torch.zeros((), dtype=q.dtype))
+        o[:, hd] = ((q[:, hd] @ k[:, hd].T) * mask) @ v[:, hd]
+    return o
+
+
+def sigmoid_weighted_sum(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, temp: torch.Tensor,
+                         bias: torch.Tensor) -> torch.Tensor:
+    """o_i = sum_{j <= i} sigmoid((q_i . k_j) scale temp_h + bias_h) v_j; q [T, H, d], k [T, G, d], v [T, G, dv]."""
+    T, H, _ = q.shape
+    rep = H // k.shape[1]
+    visible = torch.tril(torch.ones(T, T, dtype=torch.bool))
+    o = torch.zeros(T, H, v.shape[-1], dtype=q.dtype)
+    for hd in range(H):
+        s = (q[:, hd] @ k[:, hd // rep].T) * scale * temp[hd]
+        o[:, hd] = (torch.sigmoid(s + bias[hd]) * visible) @ v[:, hd // rep]
+    return o
+
+
 def gated_linear_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: dict) -> torch.Tensor:
-    """S_t = diag(a_t) S_{t-1} + k_t v_t^T, o_t = S_t^T q_t per head, written as the explicit double sum
-    o_t = sum_{s <= t} (sum_i q_t[i] k_s[i] prod_{s < r <= t} a_r[i]) v_s."""
     T = h.shape[0]
     H, d, dv = m["heads"], m["dim"], m["vdim"]
     q = (h @ w[p + "q"].T).view(T, H, d) * d ** -0.5
     k = (h @ w[p + "k"].T).view(T, H, d)
     v = (h @ w[p + "v"].T).view(T, H, dv)
     z = (h @ w[p + "a1"].T) @ w[p + "a2"].T + w[p + "a2.b"]
-    la = (torch.nn.functional.logsigmoid(z) / m["tau"]).view(T, H, d)
-    cum = la.cumsum(0)                                                        # log of the decay from the start to t
-    o = torch.zeros(T, H, dv, dtype=h.dtype)
-    for t in range(T):
-        wgt = torch.exp(cum[t][None] - cum[: t + 1])                          # [s, H, d]: prod_{s < r <= t} a_r
-        score = (q[t][None] * k[: t + 1] * wgt).sum(-1)                       # [s, H]
-        o[t] = torch.einsum("sh,shv->hv", score, v[: t + 1])
-    o = unit_rms(o, m["eps"]) * w[p + "norm"]
+    log_a = (torch.nn.functional.logsigmoid(z) / m["tau"]).view(T, H, d)
+    o = unit_rms(decayed_sum_per_channel(q, k, v, log_a), m["eps"]) * w[p + "norm"]
     return (o.reshape(T, H * dv) * silu(h @ w[p + "g"].T)) @ w[p + "o"].T
 
 
 def sigmoid_attention(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: dict) -> torch.Tensor:
-    """Causal attention whose weights are sigmoid(score + bias_h), not normalised; the values are the keys as projected."""
+    """The values are the keys as projected: before their norm and rotation."""
     T = h.shape[0]
-    H, G, d = m["heads"], m["kv_heads"], m["dim"]
+    H, G, d = m["heads"], m.get("kv_heads", m["heads"]), m["dim"]
     rot = m.get("rot") or {"dims": 0, "base": 1.0}
     q = (h @ w[p + "q"].T).view(T, H, d)
     k = (h @ w[p + "k"].T).view(T, G, d)
-    v = k
     qn = rotate_pairs(unit_rms(q, m["eps"]) * w[p + "q.norm"], rot["dims"], rot["base"], True)
     kn = rotate_pairs(unit_rms(k, m["eps"]) * w[p + "k.norm"], rot["dims"], rot["base"], True)
-    rep = H // G
-    o = torch.zeros(T, H, d, dtype=h.dtype)
-    visible = torch.tril(torch.ones(T, T, dtype=torch.bool))
-    for hd in range(H):
-        s = (qn[:, hd] @ kn[:, hd // rep].T) * m["scale"] * w[p + "temp"][hd]
-        wt = torch.sigmoid(s + w[p + "pb"][hd]) * visible
-        o[:, hd] = wt @ v[:, hd // rep]
+    o = sigmoid_weighted_sum(qn, kn, k, m["scale"], w[p + "temp"], w[p + "pb"])
     return o.reshape(T, H * d) @ w[p + "o"].T
 
 
 def retention(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: dict) -> torch.Tensor:
-    """o_t = sum_{s <= t} g^(t - s) (q_t . k_s) v_s per head, g the head's fixed decay."""
     T = h.shape[0]
     H, d, dv = m["heads"], m["dim"], m["vdim"]
     rot = m.get("rot") or {"dims": 0, "base": 1.0}
     q = rotate_pairs((h @ w[p + "q"].T).view(T, H, d), rot["dims"], rot["base"], False)
     k = rotate_pairs((h @ w[p + "k"].T).view(T, H, d), rot["dims"], rot["base"], False) * d ** -0.5
     v = (h @ w[p + "v"].T).view(T, H, dv)
-    t = torch.arange(T, dtype=h.dtype)
-    dist = t[:, None] - t[None, :]
-    o = torch.zeros(T, H, dv, dtype=h.dtype)
-    for hd in range(H):
-        g = torch.tensor(m["decay"][hd], dtype=h.dtype)
-        mask = torch.where(dist >= 0, g ** dist.clamp_min(0), torch.zeros((), dtype=h.dtype))
-        o[:, hd] = ((q[:, hd] @ k[:, hd].T) * mask) @ v[:, hd]
-    o = unit_rms(o, m["eps"])
+    o = unit_rms(decayed_sum_per_head(q, k, v, m["decay"]), m["eps"])
     return (o.reshape(T, H * dv) * silu(h @ w[p + "g"].T)) @ w[p + "o"].T
 
 
@@ -136,7 +152,8 @@ def route(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, r: dict):
     s = torch.sigmoid(h @ w[p + "router"].T)
     choice = s + w[p + "correction"]
     E, top = r["experts"], r["top"]
-    gc, keep = r["groups"]["count"], r["groups"]["keep"]
+    groups = r.get("groups") or {"count": 1, "keep": 1}
+    gc, keep = groups["count"], groups["keep"]
     per = E // gc
     chosen, weights = [], []
     for t in range(h.shape[0]):
@@ -150,7 +167,7 @@ def route(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, r: dict):
         ids = sorted(allowed, key=lambda e: (-c[e], e))[:top]
         tot = sum(float(s[t, e]) for e in ids) + 1e-20
         chosen.append(ids)
-        weights.append([float(s[t, e]) / tot * r["scale"] for e in ids])
+        weights.append([float(s[t, e]) / tot * r.get("scale", 1.0) for e in ids])
     return chosen, weights
 
 
@@ -185,8 +202,20 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], dtyp
         x = group_rms_norm(c * x + MIXERS[spec["type"]](x, w, p + "mix.", m), w[p + "norm1"], groups, eps)
         if spec.get("mlp") is not None:
             x = group_rms_norm(c * x + mixture_of_experts(x, w, p + "mlp.", spec["mlp"]), w[p + "norm2"], groups, eps)
+        elif p + "norm2" in w:
+            x = group_rms_norm(c * x, w[p + "norm2"], groups, eps)
         if side:
             x = token_side(x, tokens, w, i, side["dim"], eps)
         if streams is not None:
             streams.append(x.clone())
     return group_rms_norm(x, w["final.norm"], groups, eps) @ w["head"].T
+
+
+def greedy(cfg: dict, weights: Dict[str, torch.Tensor], tokens: List[int], n: int) -> List[int]:
+    """n tokens generated greedily, every step a whole-sequence forward."""
+    toks, out = list(tokens), []
+    for _ in range(n):
+        nxt = int(forward(cfg, weights, toks)[-1].argmax())
+        out.append(nxt)
+        toks.append(nxt)
+    return out
