@@ -102,7 +102,7 @@ def test_equal_and_unit_sizes():
     of 1, a layer without feed-forward that still has its second norm, no side input, width equal to the vocabulary."""
     layers = [(vu.attention(heads=2, kv_heads=2, dim=8, rot_dims=8), vu.moe(experts=3, top=1, count=1, keep=1, ff=8)),
               (vu.retention(heads=1, dim=4, vdim=4, rot_dims=0, decay=(1.0,)), None),
-              (vu.gla(heads=1, dim=4, vdim=4, tau=1.0, rank=1), vu.moe(experts=4, top=4, count=4, keep=4, ff=4, scale=1.0)),
+              (vu.gla(heads=1, dim=8, vdim=8, tau=1.0, rank=1), vu.moe(experts=4, top=4, count=4, keep=4, ff=4, scale=1.0)),
               (vu.attention(heads=3, kv_heads=1, dim=4, rot_dims=0), None)]
     cfg = vu.make_config(layers=layers, width=16, vocab=16, groups=1, alpha=1.0, side=0)
     w = vu.make_weights(cfg, seed=11, norm2_without_mlp=True)

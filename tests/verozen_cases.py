@@ -55,6 +55,10 @@ def check_group_norm(ops, device, dtype, T=7, D=48, groups=3, alpha=2.5, eps=1e-
     _close(xd, x.double() + ref.unit_rms(y, eps) * w, 2e-6, "the normed residual add")
 
 
+# an angle of 700 radians held in fp32 (frequencies rounded to fp32, then the product) is good to about 5e-5 radians
+ROT32 = 1e-4
+
+
 def check_head_norm_rope(ops, device, dtype, interleaved, rot_dims, d=24, H=3, with_norm=True, scale=0.5, base=37.0, eps=1e-5):
     g = torch.Generator().manual_seed(1)
     T = 9
@@ -75,12 +79,12 @@ def check_head_norm_rope(ops, device, dtype, interleaved, rot_dims, d=24, H=3, w
         got = ops.head_norm_rope(view, _dev(w.to(dtype), device) if with_norm else None, eps, positions.to(device), inv_freq,
                                  rot_dims, interleaved, scale, out_dtype)
         assert got.dtype == out_dtype
-        _close(got, want, _tol(dtype) if out_dtype != torch.float32 else 3e-5, f"rotation, pairs {'2i,2i+1' if interleaved else 'i,i+n/2'}")
+        _close(got, want, _tol(dtype) if out_dtype != torch.float32 else ROT32, f"rotation, pairs {'2i,2i+1' if interleaved else 'i,i+n/2'}")
     cache = torch.zeros(40, H, d, dtype=dtype, device=device)
     loc = torch.tensor([7, 3, 39, 1, 2, 20, 21, 8, 9], dtype=torch.int64, device=device)
     ops.head_norm_rope(view, _dev(w.to(dtype), device) if with_norm else None, eps, positions.to(device), inv_freq, rot_dims,
                        interleaved, scale, dtype, cache=cache, loc=loc)
-    _close(cache[loc], want, _tol(dtype), "rows written into the cache")
+    _close(cache[loc], want, max(_tol(dtype), ROT32), "rows written into the cache")
     assert float(cache[0].abs().max()) == 0.0
 
 
@@ -187,7 +191,7 @@ class KVSetup:
         T, G, d = kn.shape
         g = torch.Generator().manual_seed(seed)
         self.tab = Table(device)
-        n_slots = T + 70
+        n_slots = T + 70 if page == 1 else (T // page + 4) * page
         if page == 1:
             slots = torch.randperm(n_slots - 1, generator=g)[:T] + 1
         else:
@@ -294,8 +298,11 @@ def check_experts(ops, device, dtype, T=37, D=48, ff=40, E=5, top=2):
     up = _bf(torch.randn(E, ff, D, generator=g) * D ** -0.5)
     down = _bf(torch.randn(E, D, ff, generator=g) * ff ** -0.5)
     ids = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).to(torch.int32)
-    ids[:5] = torch.tensor([3, 0][:top], dtype=torch.int32)         # a crowded expert and, below, an idle one
-    ids[ids == 4] = 1
+    if E > top:                                                     # an idle expert: its pairs go to the one before it
+        ids[ids == E - 1] = -1
+        for t in range(T):
+            if -1 in ids[t].tolist():
+                ids[t][ids[t] == -1] = [e for e in range(E - 1) if e not in ids[t].tolist()][0]
     plan = ops.moe_align(ids.to(device), E)
     a = ops.moe_grouped_linear(h.to(dtype).to(device), up.to(dtype).to(device), plan, gather=True, gelu=True)
     y = ops.moe_grouped_linear(a, down.to(dtype).to(device), plan, gather=False, gelu=False)

@@ -36,8 +36,11 @@ def make_config(layers=None, width=48, vocab=53, groups=3, alpha=2.0, side=6, ep
     return cfg
 
 
-def make_weights(cfg, seed=0, norm2_without_mlp=False):
-    """Checkpoint-named tensors with bf16-representable values, so that a bf16 and an fp32 run read the same numbers."""
+def make_weights(cfg, seed=0, norm2_without_mlp=False, separated_router=False):
+    """Checkpoint-named tensors with bf16-representable values, so that a bf16 and an fp32 run read the same numbers.
+    separated_router: the selection corrections lie 1.5 apart in a shuffled order, so that no rounding of the scores (which
+    lie in (0, 1)) can change which experts are chosen -- a bf16 run against a float64 oracle would otherwise rest on close
+    calls; the experts' weights still depend on the token."""
     g = torch.Generator().manual_seed(seed)
     D, V, L = cfg["width"], cfg["vocab"], len(cfg["layers"])
 
@@ -73,6 +76,8 @@ def make_weights(cfg, seed=0, norm2_without_mlp=False):
             w[p + "norm2"] = rnd(D, std=0.1, mean=1.0)
             w[p + "mlp.router"] = rnd(E, D, std=2.0 * D ** -0.5)
             w[p + "mlp.correction"] = rnd(E, std=0.5, mean=-0.5)        # selection scores of both signs
+            if separated_router:
+                w[p + "mlp.correction"] = ((torch.randperm(E, generator=g).float() - E / 2) * 1.5).to(torch.bfloat16)
             for e in range(E):
                 w[f"{p}mlp.e{e}.up"], w[f"{p}mlp.e{e}.down"] = rnd(ff, D, std=D ** -0.5), rnd(D, ff, std=ff ** -0.5)
         elif norm2_without_mlp:
