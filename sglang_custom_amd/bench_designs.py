@@ -225,3 +225,204 @@ def run(size: str, dtype: str = "bfloat16", steps: int = 32, prefill_bs: int = 4
     out["stream_kernels_decode"] = stream_kernels(s, decode_bs)
     out["stream_kernels_prefill"] = stream_kernels(s, prefill_bs * prefill_len)
     return out
+
+
+# ------------------------------------------------------------------------------------------------ Verozen beside Llama
+# Verozen is compared with the package's closest model, Llama (multi-head attention with grouped key / value heads over
+# per-head keys and values, RMS norms, one residual stream): same width, depth, vocabulary, attention heads and head
+# width; Llama's dense feed-forward is as wide as the experts one Verozen token uses together.
+VEROZEN_SIZES = {
+    "vz2048": dict(width=2048, heads=16, kv_heads=4, dim=128, rec_heads=16, rec_dim=64, rec_vdim=128, experts=32, top=4, groups=4,
+                   keep=2, ff=2048, layers=4, vocab=32768, side=64, norm_groups=8, gate_rank=64),
+    "vz4096": dict(width=4096, heads=32, kv_heads=8, dim=128, rec_heads=32, rec_dim=64, rec_vdim=128, experts=64, top=8, groups=8,
+                   keep=4, ff=1536, layers=4, vocab=32768, side=64, norm_groups=8, gate_rank=64),
+    "vztiny": dict(width=256, heads=8, kv_heads=2, dim=64, rec_heads=4, rec_dim=32, rec_vdim=64, experts=8, top=2, groups=4, keep=2,
+                   ff=128, layers=3, vocab=2048, side=16, norm_groups=4, gate_rank=16),
+}
+
+
+def verozen_config(s: dict) -> dict:
+    mlp = dict(kind="moe", expert=dict(ff=s["ff"]),
+               router=dict(experts=s["experts"], top=s["top"], scale=1.0, groups=dict(count=s["groups"], keep=s["keep"])))
+    gla = dict(type="gla", mixer=dict(heads=s["rec_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"], tau=16.0, gate_rank=s["gate_rank"]), mlp=mlp)
+    att = dict(type="attention", mixer=dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5,
+                                            rot=dict(base=500000.0, dims=s["dim"] // 2)), mlp=mlp)
+    ret = dict(type="retention", mixer=dict(heads=s["rec_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"],
+                                            decay=[1.0 - 2.0 ** (-5 - (i % 6)) for i in range(s["rec_heads"])],
+                                            rot=dict(base=1000000.0, dims=s["rec_dim"])), mlp=mlp)
+    order = [gla, att, ret, gla]
+    return dict(architecture="Verozen", vocab=s["vocab"], width=s["width"], postln_alpha=3.0, norm=dict(eps=1e-5, groups=s["norm_groups"]),
+                token_side=dict(dim=s["side"]), layers=[order[i % 4] for i in range(s["layers"])])
+
+
+def llama_config(s: dict, dtype: str) -> dict:
+    return dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=s["width"], num_hidden_layers=s["layers"],
+                num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], head_dim=s["dim"],
+                intermediate_size=s["ff"] * s["top"], vocab_size=s["vocab"], rms_norm_eps=1e-5, rope_theta=500000.0,
+                max_position_embeddings=16384, rope_scaling=None, tie_word_embeddings=False, torch_dtype=dtype, hidden_act="silu",
+                attention_bias=False, mlp_bias=False)
+
+
+def verozen_mixer_kernels(s: dict, bs: int, ctx: int, prefill_bs: int, prefill_len: int) -> dict:
+    """The token mixers' launches alone, bf16, beside Llama's attention launches on the same heads.  Decode attention:
+    bytes = every visible key and value row once per sequence.  Prefill attention: flops 2 (d + dv) per causal
+    query-key pair and head.  The recurrence has no like kernel in the package: a decode step is priced by the bytes of
+    the matrices it must read and write, a prefill by the fp32 vector flops it does (6 per matrix element and token)."""
+    from . import ops
+
+    dev, dt = "cuda", torch.bfloat16
+    H, G, d = s["heads"], s["kv_heads"], s["dim"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    res = {}
+    # ---- decode attention
+    slots = bs * ctx + 8
+    kc = torch.randn(slots, G, d, device=dev, generator=g).to(dt)
+    vc = torch.randn(slots, G, d, device=dev, generator=g).to(dt)
+    rtt = (torch.arange(bs * ctx, device=dev, dtype=torch.int32) + 1).view(bs, ctx)
+    rpi = torch.arange(bs, device=dev)
+    q = torch.randn(bs, H, d, device=dev, generator=g).to(dt)
+    o = torch.empty_like(q)
+    temp, bias = torch.ones(H, device=dev), torch.full((H,), -4.0, device=dev)
+    pos = torch.full((bs,), ctx - 1, device=dev, dtype=torch.int64)
+    splits = ops.sigmoid_attention_splits(bs, H, G, ctx, dt)
+    t = _timed(lambda: ops.sigmoid_attention(q, kc, vc, o, rtt, rpi, pos, temp, bias, d ** -0.5, num_splits=splits), 20)
+    b = bs * ctx * G * d * 2 * 2
+    res["verozen_decode_attention"] = dict(us=round(t * 1e6, 1), splits=splits, gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
+    seq = torch.full((bs,), ctx, device=dev, dtype=torch.int64)
+    nsp = int(ops.decode_num_splits(bs, G, ctx, 64))
+    logits = torch.empty(bs * H * nsp * d, device=dev, dtype=torch.float32)
+    lse = torch.empty(bs * H * nsp, device=dev, dtype=torch.float32)
+    o2 = torch.empty(bs, H, d, device=dev, dtype=dt)
+    t = _timed(lambda: ops.decode_attention_paged(q, kc, vc, o2, rtt, rpi, seq, logits if nsp > 1 else None, lse if nsp > 1 else None,
+                                                  nsp, d ** -0.5), 20)
+    res["llama_decode_attention"] = dict(us=round(t * 1e6, 1), splits=nsp, gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
+    # ---- prefill attention
+    T = prefill_bs * prefill_len
+    kp = torch.randn(T + 8, G, d, device=dev, generator=g).to(dt)
+    vp = torch.randn(T + 8, G, d, device=dev, generator=g).to(dt)
+    rtp = (torch.arange(T, device=dev, dtype=torch.int32) + 1).view(prefill_bs, prefill_len)
+    qp = torch.randn(T, H, d, device=dev, generator=g).to(dt)
+    op = torch.empty_like(qp)
+    posp = torch.arange(prefill_len, device=dev).repeat(prefill_bs)
+    tok_req = torch.repeat_interleave(torch.arange(prefill_bs, device=dev, dtype=torch.int32), prefill_len)
+    bq = ops.sigmoid_attention_block_tokens(H, G, dt)
+    assert prefill_len % bq == 0
+    starts = torch.arange(0, T, bq, dtype=torch.int32)
+    blocks = torch.stack([starts, torch.full_like(starts, bq)], 1).to(dev)
+    t = _timed(lambda: ops.sigmoid_attention(qp, kp, vp, op, rtp, torch.arange(prefill_bs, device=dev), posp, temp, bias, d ** -0.5,
+                                             tok_req=tok_req, blocks=blocks), 3)
+    pairs = prefill_bs * prefill_len * (prefill_len + 1) // 2
+    fl = pairs * H * 2 * 2 * d
+    res["verozen_prefill_attention"] = dict(ms=round(t * 1e3, 3), tflops=round(fl / t / 1e12, 1), of_mfma_peak=round(fl / t / MFMA_BF16_PEAK, 3))
+    km = torch.randn(T, G, d, device=dev, generator=g).to(dt)
+    vm = torch.randn(T, G, d, device=dev, generator=g).to(dt)
+    qo = torch.arange(0, T + 1, prefill_len, device=dev, dtype=torch.int32)
+    kvp = torch.zeros(prefill_bs + 1, device=dev, dtype=torch.int32)
+    dummy = torch.zeros(1, device=dev, dtype=torch.int32)
+    t = _timed(lambda: ops.extend_attention_fwd(qp, km, vm, op, km, vm, qo, kvp, dummy, None, True, None, prefill_len, d ** -0.5, 0.0), 5)
+    res["llama_prefill_attention"] = dict(ms=round(t * 1e3, 3), tflops=round(fl / t / 1e12, 1), of_mfma_peak=round(fl / t / MFMA_BF16_PEAK, 3))
+    # ---- the recurrence
+    RH, dk, dv = s["rec_heads"], s["rec_dim"], s["rec_vdim"]
+    state = torch.zeros(bs + 1, RH, dk, dv, device=dev)
+    r2s = torch.arange(1, bs + 1, device=dev, dtype=torch.int32)
+    for name, gated in (("gla", True), ("retention", False)):
+        qk_dt = dt if gated else torch.float32
+        qd = torch.randn(bs, RH, dk, device=dev, generator=g).to(qk_dt)
+        kd = torch.randn(bs, RH, dk, device=dev, generator=g).to(qk_dt)
+        vd = torch.randn(bs, RH, dv, device=dev, generator=g).to(dt)
+        od = torch.empty(bs, RH, dv, device=dev)
+        z = torch.randn(bs, RH * dk, device=dev, generator=g) if gated else None
+        hd = None if gated else torch.full((RH,), 0.99, device=dev)
+        posd = torch.full((bs,), ctx, device=dev, dtype=torch.int64)
+        t = _timed(lambda: ops.linear_recurrence(qd, kd, vd, od, state, r2s, rpi, posd, 1.0, gate_logits=z, tau=16.0, head_decay=hd), 20)
+        b = bs * RH * dk * dv * 4 * 2
+        res[f"verozen_{name}_decode_recurrence"] = dict(us=round(t * 1e6, 1), gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
+        qd = torch.randn(T, RH, dk, device=dev, generator=g).to(qk_dt)
+        kd = torch.randn(T, RH, dk, device=dev, generator=g).to(qk_dt)
+        vd = torch.randn(T, RH, dv, device=dev, generator=g).to(dt)
+        od = torch.empty(T, RH, dv, device=dev)
+        z = torch.randn(T, RH * dk, device=dev, generator=g) if gated else None
+        ss = torch.arange(0, T, prefill_len, device=dev, dtype=torch.int32)
+        sl = torch.full((prefill_bs,), prefill_len, device=dev, dtype=torch.int32)
+        t = _timed(lambda: ops.linear_recurrence(qd, kd, vd, od, state, r2s, torch.arange(prefill_bs, device=dev), posp, 1.0,
+                                                 gate_logits=z, tau=16.0, head_decay=hd, tok_req=tok_req, seg_start=ss, seg_len=sl), 3)
+        fl = T * RH * dk * dv * 6
+        res[f"verozen_{name}_prefill_recurrence"] = dict(ms=round(t * 1e3, 3), vector_tflops=round(fl / t / 1e12, 2),
+                                                          tokens_per_s_per_sequence=round(prefill_len / t))
+    return res
+
+
+def verozen_ff_and_stream_kernels(s: dict, tokens: int) -> dict:
+    """The mixture's launches beside Llama's dense feed-forward GEMMs at equal flops per token, and the post-norm
+    launches beside fused_add_rmsnorm by bytes moved (bf16 activations)."""
+    import torch.nn.functional as F
+
+    from . import ops
+
+    dev, dt = "cuda", torch.bfloat16
+    D, ff, E, top = s["width"], s["ff"], s["experts"], s["top"]
+    g = torch.Generator(device=dev).manual_seed(0)
+    res = {}
+    x = torch.randn(tokens, D, device=dev, generator=g)
+    h = x.to(dt)
+    wr = torch.randn(E, D, device=dev, generator=g) * D ** -0.5
+    corr = torch.zeros(E, device=dev)
+    up = (torch.randn(E, ff, D, device=dev, generator=g) * D ** -0.5).to(dt)
+    down = (torch.randn(E, D, ff, device=dev, generator=g) * ff ** -0.5).to(dt)
+    logits = ops.linear(x, wr)
+    t = _timed(lambda: ops.linear(x, wr), 10)
+    res["router_logits_fp32"] = dict(us=round(t * 1e6, 1))
+    ids, wts = ops.moe_route_grouped(logits, corr, top, s["groups"], s["keep"], 1.0)
+    t = _timed(lambda: ops.moe_route_grouped(logits, corr, top, s["groups"], s["keep"], 1.0), 10)
+    res["moe_route_grouped"] = dict(us=round(t * 1e6, 1))
+    plan = ops.moe_align(ids, E)
+    t = _timed(lambda: ops.moe_align(ids, E), 10)
+    res["moe_align"] = dict(us=round(t * 1e6, 1))
+    a = ops.moe_grouped_linear(h, up, plan, gather=True, gelu=True)
+    t1 = _timed(lambda: ops.moe_grouped_linear(h, up, plan, gather=True, gelu=True), 5)
+    t2 = _timed(lambda: ops.moe_grouped_linear(a, down, plan, gather=False, gelu=False), 5)
+    fl = tokens * top * 2 * ff * D
+    wbytes = E * ff * D * 2
+    res["moe_up_gelu"] = dict(us=round(t1 * 1e6, 1), tflops=round(fl / t1 / 1e12, 1), of_mfma_peak=round(fl / t1 / MFMA_BF16_PEAK, 3),
+                              weight_gbs=round(wbytes / t1 / 1e9))
+    res["moe_down"] = dict(us=round(t2 * 1e6, 1), tflops=round(fl / t2 / 1e12, 1), of_mfma_peak=round(fl / t2 / MFMA_BF16_PEAK, 3),
+                           weight_gbs=round(wbytes / t2 / 1e9))
+    # the closest model's feed-forward: one [ff * top, D] up projection (half of gate_up) and the down projection
+    wu = (torch.randn(ff * top, D, device=dev, generator=g) * D ** -0.5).to(dt)
+    wd = (torch.randn(D, ff * top, device=dev, generator=g) * (ff * top) ** -0.5).to(dt)
+    mid = torch.randn(tokens, ff * top, device=dev, generator=g).to(dt)
+    t1 = _timed(lambda: F.linear(h, wu), 5)
+    t2 = _timed(lambda: F.linear(mid, wd), 5)
+    res["dense_up (closest, library GEMM)"] = dict(us=round(t1 * 1e6, 1), tflops=round(fl / t1 / 1e12, 1), of_mfma_peak=round(fl / t1 / MFMA_BF16_PEAK, 3),
+                                                    weight_gbs=round(ff * top * D * 2 / t1 / 1e9))
+    res["dense_down (closest, library GEMM)"] = dict(us=round(t2 * 1e6, 1), tflops=round(fl / t2 / 1e12, 1), of_mfma_peak=round(fl / t2 / MFMA_BF16_PEAK, 3),
+                                                      weight_gbs=round(ff * top * D * 2 / t2 / 1e9))
+    # norms
+    w = torch.ones(D, device=dev, dtype=dt)
+    y = torch.randn(tokens, D, device=dev, generator=g).to(dt)
+    t = _timed(lambda: ops.scaled_add_group_rmsnorm(x, y, 3.0, w, s["norm_groups"], 1e-5), 20)
+    res["scaled_add_group_rmsnorm"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 2 + 4 + 2) / t / 1e9))
+    yy = ops.moe_grouped_linear(a, down, plan, gather=False, gelu=False)
+    t = _timed(lambda: ops.scaled_add_group_rmsnorm(x, yy, 3.0, w, s["norm_groups"], 1e-5, rows=plan.rows, coef=wts), 20)
+    res["scaled_add_group_rmsnorm (sum of experts)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 2 * top + 4 + 2) / t / 1e9))
+    t = _timed(lambda: ops.rmsnorm_residual_add(x, y, w, 1e-5), 20)
+    res["rmsnorm_residual_add"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * (4 + 2 + 4 + 2) / t / 1e9))
+    xb, rb = x.to(dt), x.to(dt)
+    t = _timed(lambda: ops.fused_add_rmsnorm(xb, rb, w, 1e-5), 20)
+    res["fused_add_rmsnorm (closest)"] = dict(us=round(t * 1e6, 1), gbs=round(tokens * D * 2 * 4 / t / 1e9))
+    return res
+
+
+def run_verozen(size: str, dtype: str = "bfloat16", steps: int = 32, prefill_bs: int = 4, prefill_len: int = 2048, decode_bs: int = 64,
+                decode_ctx: int = 1024) -> dict:
+    s = VEROZEN_SIZES[size]
+    if size == "vztiny":
+        prefill_bs, prefill_len, decode_bs, decode_ctx = 2, 256, 8, 128
+    out = dict(size=size, shape=s, dtype=dtype, data="synthetic", workload=dict(prefill=[prefill_bs, prefill_len], decode=[decode_bs, decode_ctx], steps=steps))
+    out["verozen"] = model_throughput(verozen_config(s), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=False)
+    out["llama"] = model_throughput(llama_config(s, dtype), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=True)
+    out["llama_eager"] = model_throughput(llama_config(s, dtype), dtype, prefill_bs, prefill_len, decode_bs, decode_ctx, steps, graph=False)
+    out["mixers"] = verozen_mixer_kernels(s, decode_bs, decode_ctx, prefill_bs, prefill_len)
+    out["ff_and_stream_decode"] = verozen_ff_and_stream_kernels(s, decode_bs)
+    out["ff_and_stream_prefill"] = verozen_ff_and_stream_kernels(s, prefill_bs * prefill_len)
+    return out

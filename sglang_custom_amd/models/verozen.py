@@ -306,7 +306,9 @@ class VerozenForCausalLM(nn.Module):
     @torch.no_grad()
     def init_random_weights(self, seed: int = 0, std: float = 0.02) -> None:
         if self.model is None:
-            self._build(norm2_layers=())
+            # without a checkpoint the decay projection's rank is the configuration's optional "gate_rank", or the default
+            self._build(norm2_layers=(), gate_ranks={i: int(spec["mixer"]["gate_rank"]) for i, spec in enumerate(self.config.layer_specs)
+                                                     if spec["type"] == "gla" and spec["mixer"].get("gate_rank")})
         dev = self.lm_head.weight.device
         g = torch.Generator(device=dev).manual_seed(seed)
         for name, p in self.named_parameters():
