@@ -750,33 +750,36 @@ int mi355_linear_recurrence(float* out, float* state, const void* q, const void*
  *   req_to_token.  `blocks` lists runs (first token, count <= mi355_sigmoid_attention_block_tokens(...)) of consecutive
  *   tokens of one sequence; null = one token per run and num_blocks = tokens, and then num_splits > 1 cuts every token's
  *   keys into that many ranges whose partial sums (split_scratch: num_splits * tokens * heads * v_head_dim floats) a second
- *   launch adds.  The new tokens' keys and values must be in the caches already. */
-int mi355_sigmoid_attention_block_tokens(int heads, int kv_heads, int dtype);
+ *   launch adds.  max_run: the longest run in `blocks` (1 without).  The new tokens' keys and values must be in the
+ *   caches already. */
+int mi355_sigmoid_attention_block_tokens(int heads, int kv_heads, int head_dim, int v_head_dim, int dtype);
 int mi355_sigmoid_attention(void* out, const void* q, const void* k_cache, const void* v_cache, const int32_t* req_to_token,
                             const int64_t* req_pool_indices, const int32_t* tok_req, const int64_t* positions,
                             const int32_t* blocks, int64_t num_blocks, const float* temp, const float* bias,
                             int64_t q_token_stride, int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride,
                             int64_t req_to_token_stride, int heads, int kv_heads, int head_dim, int v_head_dim, float scale,
-                            int num_splits, float* split_scratch, int64_t tokens, int dtype, void* stream);
+                            int num_splits, float* split_scratch, int64_t tokens, int max_run, int dtype, void* stream);
 
 /* ---- mixture of experts ------------------------------------------------------------------------------
  * mi355_moe_route_grouped: s = sigmoid(logits) (fp32 [tokens, num_experts]); selection on s + correction: experts form
  *   n_groups equal groups of neighbours, a group scores the sum of its two largest selection scores (its only one, for
  *   groups of one), the keep_groups best groups stay, the `top` largest selection scores among them are chosen (ties: the
  *   smaller index); weights[t][k] = s[chosen] / (sum of the chosen s + 1e-20) * scale.
- * mi355_moe_align: sorts the tokens * top (token, choice) pairs by expert into blocks of mi355_moe_block_rows() rows of
- *   one expert each: src_row[p] = token of sorted row p or -1 (padding), rows[pair] = p, tile_expert[block] = its expert,
+ * mi355_moe_router_logits: out[t][j] = x[t] . weight[j] in exact fp32 for few rows (one wave per row; k <= 8192).
+ * mi355_moe_align: sorts the tokens * top (token, choice) pairs by expert into blocks of `block` rows
+ *   (mi355_moe_block_rows(0), or mi355_moe_block_rows(1) for prefill-sized steps of 16-bit models) of one expert each: src_row[p] = token of sorted row p or -1 (padding), rows[pair] = p, tile_expert[block] = its expert,
  *   *n_tiles = blocks in use.  `padded` (a multiple of the block) must be at least pairs + min(experts, pairs) * (block - 1).
  * mi355_moe_grouped_linear: out[p][.] = act(weight[tile_expert[p / block]] . in[gather ? src_row[p] : p]) for every sorted
  *   row p of a block in use (0 for padding rows); weight [experts, n, k]; act = erf-GELU when `gelu`. */
 int mi355_moe_route_grouped(int32_t* ids, float* weights, const float* logits, const float* correction, int64_t tokens,
                             int num_experts, int top, int n_groups, int keep_groups, float scale, void* stream);
-int mi355_moe_block_rows(void);
+int mi355_moe_block_rows(int wide);
+int mi355_moe_router_logits(float* out, const float* x, const float* weight, int64_t rows, int n, int k, void* stream);
 int mi355_moe_align(int32_t* src_row, int32_t* rows, int32_t* tile_expert, int32_t* n_tiles, const int32_t* ids, int64_t tokens,
-                    int top, int num_experts, int64_t padded, void* stream);
+                    int top, int num_experts, int block, int64_t padded, void* stream);
 int mi355_moe_grouped_linear(void* out, const void* in, int64_t in_stride, const void* weight, const int32_t* src_row,
-                             const int32_t* tile_expert, const int32_t* n_tiles, int gather, int gelu, int64_t padded, int n, int k,
-                             int dtype, void* stream);
+                             const int32_t* tile_expert, const int32_t* n_tiles, int gather, int gelu, int64_t padded, int block,
+                             int n, int k, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -109,12 +109,13 @@ _SIGNATURES = {
     "mi355_head_rmsnorm_gate": (I, [P, P, P, P, L, L, I, I, F, I, P]),
     "mi355_gelu_tanh_mul_rows": (I, [P, P, L, P, L, L, L, P, L, L, I, P]),
     "mi355_linear_recurrence": (I, [P, P, P, P, P, P, P, P, P, P, P, P, P, L, I, I, I, L, L, L, L, F, F, I, I, P]),
-    "mi355_sigmoid_attention_block_tokens": (I, [I, I, I]),
-    "mi355_sigmoid_attention": (I, [P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, I, I, I, I, F, I, P, L, I, P]),
+    "mi355_sigmoid_attention_block_tokens": (I, [I, I, I, I, I]),
+    "mi355_sigmoid_attention": (I, [P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, I, I, I, I, F, I, P, L, I, I, P]),
     "mi355_moe_route_grouped": (I, [P, P, P, P, L, I, I, I, I, F, P]),
-    "mi355_moe_block_rows": (I, []),
-    "mi355_moe_align": (I, [P, P, P, P, P, L, I, I, L, P]),
-    "mi355_moe_grouped_linear": (I, [P, P, L, P, P, P, P, I, I, L, I, I, I, P]),
+    "mi355_moe_block_rows": (I, [I]),
+    "mi355_moe_router_logits": (I, [P, P, P, L, I, I, P]),
+    "mi355_moe_align": (I, [P, P, P, P, P, L, I, I, I, L, P]),
+    "mi355_moe_grouped_linear": (I, [P, P, L, P, P, P, P, I, I, L, I, I, I, I, P]),
     "mi355_latent_window_attention": (I, [P, P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, L, L, L, I, I, I, I, I, F, I, P, L, I, P]),
 }
 

@@ -305,12 +305,12 @@ def verozen_mixer_kernels(s: dict, bs: int, ctx: int, prefill_bs: int, prefill_l
     op = torch.empty_like(qp)
     posp = torch.arange(prefill_len, device=dev).repeat(prefill_bs)
     tok_req = torch.repeat_interleave(torch.arange(prefill_bs, device=dev, dtype=torch.int32), prefill_len)
-    bq = ops.sigmoid_attention_block_tokens(H, G, dt)
+    bq = ops.sigmoid_attention_block_tokens(H, G, d, d, dt)
     assert prefill_len % bq == 0
     starts = torch.arange(0, T, bq, dtype=torch.int32)
     blocks = torch.stack([starts, torch.full_like(starts, bq)], 1).to(dev)
     t = _timed(lambda: ops.sigmoid_attention(qp, kp, vp, op, rtp, torch.arange(prefill_bs, device=dev), posp, temp, bias, d ** -0.5,
-                                             tok_req=tok_req, blocks=blocks), 3)
+                                             tok_req=tok_req, blocks=blocks, max_run=bq), 3)
     pairs = prefill_bs * prefill_len * (prefill_len + 1) // 2
     fl = pairs * H * 2 * 2 * d
     res["verozen_prefill_attention"] = dict(ms=round(t * 1e3, 3), tflops=round(fl / t / 1e12, 1), of_mfma_peak=round(fl / t / MFMA_BF16_PEAK, 3))
@@ -369,14 +369,14 @@ def verozen_ff_and_stream_kernels(s: dict, tokens: int) -> dict:
     corr = torch.zeros(E, device=dev)
     up = (torch.randn(E, ff, D, device=dev, generator=g) * D ** -0.5).to(dt)
     down = (torch.randn(E, D, ff, device=dev, generator=g) * ff ** -0.5).to(dt)
-    logits = ops.linear(x, wr)
-    t = _timed(lambda: ops.linear(x, wr), 10)
+    logits = ops.moe_router_logits(x, wr)
+    t = _timed(lambda: ops.moe_router_logits(x, wr), 10)
     res["router_logits_fp32"] = dict(us=round(t * 1e6, 1))
     ids, wts = ops.moe_route_grouped(logits, corr, top, s["groups"], s["keep"], 1.0)
     t = _timed(lambda: ops.moe_route_grouped(logits, corr, top, s["groups"], s["keep"], 1.0), 10)
     res["moe_route_grouped"] = dict(us=round(t * 1e6, 1))
-    plan = ops.moe_align(ids, E)
-    t = _timed(lambda: ops.moe_align(ids, E), 10)
+    plan = ops.moe_align(ids, E, wide_ok=True)
+    t = _timed(lambda: ops.moe_align(ids, E, wide_ok=True), 10)
     res["moe_align"] = dict(us=round(t * 1e6, 1))
     a = ops.moe_grouped_linear(h, up, plan, gather=True, gelu=True)
     t1 = _timed(lambda: ops.moe_grouped_linear(h, up, plan, gather=True, gelu=True), 5)

@@ -148,39 +148,48 @@ __global__ __launch_bounds__(256) void sigmoid_attention_sum_kernel(T* __restric
   }
 }
 
-// Matrix-core kernel for 16-bit dtypes, d % 32 == 0, dv % 16 == 0.  Four waves.  Per key tile of 32:
-//   S [16 rows x 32 keys]: wave w < 2 computes the 16 keys w * 16.. with d / 32 MFMA 16x16x32 (A = Q rows from LDS, B = K rows
-//   from LDS: both 16-byte fragments along d), applies the sigmoid and the causal mask in fp32 and leaves P in LDS as T;
-//   O [16 rows x dv]: wave w owns the 16-column blocks w, w + 4, ...; per block two MFMA 16x16x16 (keys 0-15, 16-31) with
-//   A = P from LDS and B = V read down a column of the V tile.
-// sm: Qs [16][d + 8] T | Ks [32][d + 8] T | Vs [32][dv + 2] T | Ps [16][32 + 8] T
-template <typename T>
+// Matrix-core kernel for 16-bit dtypes, d % 32 == 0, dv % 16 == 0.  Four waves, SGM_ROWS = 64 (token, head) rows.  Per key
+// tile of 32:
+//   S: wave w computes its 16 rows x 32 keys with 2 * d / 32 MFMA 16x16x32 (A = Q rows, B = K rows from LDS: both 16-byte
+//      fragments along d), applies the sigmoid and the causal mask in fp32 and leaves P in LDS as T;
+//   O: wave w owns CT 16-column tiles of the result for ALL row tiles, so that each V fragment (two transposed LDS reads of
+//      four keys each) is read once per workgroup; one MFMA 16x16x32 per (row tile, column tile).
+// The next tile's K and V rows are requested from global memory into registers before the current tile's products and
+// stored to LDS after them.  A decode step's run has one token: row tiles without a valid row are skipped by whole waves.
+// sm: Qs [64][d + 8] | Ks [32][d + 8] | Vs [32][dv + 8] | Ps [64][32 + 8]   (all T)
+constexpr int SGM_ROWS = 64;
+constexpr int SGM_MAXC = 4;      // 16-byte chunks of a K (V) tile per thread: d (dv) up to 256
+
+template <typename T, int CT>
 __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smraw[];
   const int d = a.d, dv = a.dv;
-  const int qld = d + 8, vld = dv + 2, pld = SG_KT + 8;
+  const int qld = d + 8, vld = dv + 8, pld = SG_KT + 8;
   T* Qs = reinterpret_cast<T*>(smraw);
-  T* Ks = Qs + SG_ROWS * qld;
+  T* Ks = Qs + SGM_ROWS * qld;
   T* Vs = Ks + SG_KT * qld;
   T* Ps = Vs + SG_KT * vld;
-  __shared__ int row_pos[SG_ROWS];
-  __shared__ float row_mul[SG_ROWS], row_add[SG_ROWS];
+  __shared__ int row_pos[SGM_ROWS];
+  __shared__ float row_mul[SGM_ROWS], row_add[SGM_ROWS];
   const int rep = a.heads / a.kv_heads;
-  const int chunks = (rep + a.heads_per_tile - 1) / a.heads_per_tile;
+  const int HR = a.heads_per_tile;
+  const int chunks = (rep + HR - 1) / HR;
   const int g = blockIdx.y / chunks, hc = blockIdx.y - g * chunks;
   const int split = blockIdx.z;
   const int64_t t0 = a.blocks != nullptr ? a.blocks[2 * blockIdx.x] : blockIdx.x;
   const int nt = a.blocks != nullptr ? a.blocks[2 * blockIdx.x + 1] : 1;
   const int b = a.tok_req != nullptr ? a.tok_req[t0] : (int)t0;
   const int32_t* table = a.req_to_token + a.req_pool_indices[b] * a.req_to_token_stride;
-  const int h0 = g * rep + hc * a.heads_per_tile;
-  const int nh = min(a.heads_per_tile, rep - hc * a.heads_per_tile);
+  const int h0 = g * rep + hc * HR;
+  const int nh = min(HR, rep - hc * HR);
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int li = lane & 15, lg = lane >> 4;
   const T* q = (const T*)a.q;
-  const int dch = d / 8;           // 16-byte chunks per row
-  for (int e = tid; e < SG_ROWS * dch; e += 256) {
+  const int dch = d / 8, vch = dv / 8;           // 16-byte chunks per row
+  const int live_rows = nt * HR;                 // rows at or past this hold no (token, head)
+  for (int e = tid; e < SGM_ROWS * dch; e += 256) {
     const int r = e / dch, ch = e - r * dch;
-    const int tl = r / a.heads_per_tile, hl = r - tl * a.heads_per_tile;
+    const int tl = r / HR, hl = r - tl * HR;
     Vec<T, 8> val;
     if (tl < nt && hl < nh) {
       val = ldvec<T, 8>(q + (t0 + tl) * a.q_token_stride + (int64_t)(h0 + hl) * a.q_head_stride + ch * 8);
@@ -190,8 +199,8 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
     }
     stvec<T, 8>(Qs + r * qld + ch * 8, val);
   }
-  if (tid < SG_ROWS) {
-    const int tl = tid / a.heads_per_tile, hl = tid - tl * a.heads_per_tile;
+  if (tid < SGM_ROWS) {
+    const int tl = tid / HR, hl = tid - tl * HR;
     const bool ok = tl < nt && hl < nh;
     row_pos[tid] = ok ? (int)a.positions[t0 + tl] : -1;
     row_mul[tid] = ok ? a.scale * a.temp[h0 + hl] : 0.f;
@@ -201,99 +210,140 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
   const int tiles = last / SG_KT + 1;
   const int per = (tiles + a.num_splits - 1) / a.num_splits;
   const int tile_lo = split * per, tile_hi = min(tiles, tile_lo + per);
-  const int nblk = dv / 16;        // 16-column blocks of the result
-  f32x4 acc[4];                    // dv <= 256: at most 4 blocks per wave
+  const int nblk = dv / 16;
+  f32x4 acc[4][CT];
 #pragma unroll
-  for (int m = 0; m < 4; ++m) acc[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+    for (int c = 0; c < CT; ++c) acc[rt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
   const T* kc = (const T*)a.k_cache;
   const T* vc = (const T*)a.v_cache;
-  const int vch = dv / 8;
   using Frag = typename Mfma<T>::frag;
-  using Frag16 = typename Mfma16<T>::frag;
+  Vec<T, 8> kreg[SGM_MAXC], vreg[SGM_MAXC];
+  auto request = [&](int tile) {
+    const int j0 = tile * SG_KT;
+#pragma unroll
+    for (int u = 0; u < SGM_MAXC; ++u) {
+      const int e = tid + 256 * u;
+      if (e < SG_KT * dch) {
+        const int kk = e / dch, ch = e - kk * dch;
+        const int j = min(j0 + kk, last);        // keys past the run's last one are masked below; any valid row will do
+        kreg[u] = ldvec<T, 8>(kc + ((int64_t)table[j] * a.kv_heads + g) * d + ch * 8);
+      }
+      if (e < SG_KT * vch) {
+        const int kk = e / vch, ch = e - kk * vch;
+        const int j = min(j0 + kk, last);
+        vreg[u] = ldvec<T, 8>(vc + ((int64_t)table[j] * a.kv_heads + g) * dv + ch * 8);
+      }
+    }
+  };
+  if (tile_lo < tile_hi) request(tile_lo);
   for (int tile = tile_lo; tile < tile_hi; ++tile) {
     const int j0 = tile * SG_KT;
-    __syncthreads();
-    for (int e = tid; e < SG_KT * dch; e += 256) {
-      const int kk = e / dch, ch = e - kk * dch;
-      const int j = min(j0 + kk, last);       // rows past the run's last key are masked below; any valid row will do
-      stvec<T, 8>(Ks + kk * qld + ch * 8, ldvec<T, 8>(kc + ((int64_t)table[j] * a.kv_heads + g) * d + ch * 8));
-    }
-    for (int e = tid; e < SG_KT * vch; e += 256) {
-      const int kk = e / vch, ch = e - kk * vch;
-      const int j = min(j0 + kk, last);
-      const Vec<T, 8> val = ldvec<T, 8>(vc + ((int64_t)table[j] * a.kv_heads + g) * dv + ch * 8);
-      T* dst = Vs + kk * vld + ch * 8;        // rows of dv + 2: only 4-byte aligned
+    __syncthreads();                             // the last tile's readers are done (and, the first time, Qs is written)
 #pragma unroll
-      for (int x = 0; x < 8; x += 2) *reinterpret_cast<Vec<T, 2>*>(dst + x) = Vec<T, 2>{{val.v[x], val.v[x + 1]}};
+    for (int u = 0; u < SGM_MAXC; ++u) {
+      const int e = tid + 256 * u;
+      if (e < SG_KT * dch) {
+        const int kk = e / dch, ch = e - kk * dch;
+        stvec<T, 8>(Ks + kk * qld + ch * 8, kreg[u]);
+      }
+      if (e < SG_KT * vch) {
+        const int kk = e / vch, ch = e - kk * vch;
+        stvec<T, 8>(Vs + kk * vld + ch * 8, vreg[u]);
+      }
     }
     __syncthreads();
-    if (wv < 2) {
-      f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
-      const int i = lane & 15, kq = lane >> 4;
+    if (tile + 1 < tile_hi) request(tile + 1);   // in flight during this tile's products
+    if (16 * wv < live_rows) {
+      f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
       for (int c = 0; c < d; c += 32) {
-        const Frag af = *reinterpret_cast<const Frag*>(Qs + i * qld + c + 8 * kq);
-        const Frag bf = *reinterpret_cast<const Frag*>(Ks + (wv * 16 + i) * qld + c + 8 * kq);
-        s = Mfma<T>::run(af, bf, s);
+        const Frag af = *reinterpret_cast<const Frag*>(Qs + (16 * wv + li) * qld + c + 8 * lg);
+        const Frag b0 = *reinterpret_cast<const Frag*>(Ks + li * qld + c + 8 * lg);
+        const Frag b1 = *reinterpret_cast<const Frag*>(Ks + (16 + li) * qld + c + 8 * lg);
+        s0 = Mfma<T>::run(af, b0, s0);
+        s1 = Mfma<T>::run(af, b1, s1);
       }
-      // result lane: rows 4 * (lane >> 4) + x, key column lane & 15
-      const int key = j0 + wv * 16 + (lane & 15);
+      // result lane: rows 16 wv + 4 lg + x, key columns li (s0) and 16 + li (s1)
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
-        const int r = 4 * (lane >> 4) + x;
-        const float p = key <= row_pos[r] ? sg_sigmoid(s[x] * row_mul[r] + row_add[r]) : 0.f;
-        Ps[r * pld + wv * 16 + (lane & 15)] = from_f32<T>(p);
+        const int r = 16 * wv + 4 * lg + x;
+        const int rp = row_pos[r];
+        const float m = row_mul[r], ad = row_add[r];
+        Ps[r * pld + li] = from_f32<T>(j0 + li <= rp ? sg_sigmoid(s0[x] * m + ad) : 0.f);
+        Ps[r * pld + 16 + li] = from_f32<T>(j0 + 16 + li <= rp ? sg_sigmoid(s1[x] * m + ad) : 0.f);
       }
     }
     __syncthreads();
     {
-      const int i = lane & 15, kq = lane >> 4;
-      Frag16 p0, p1;
-      {
-        const Vec<T, 4> x0 = ldvec<T, 4>(Ps + i * pld + 4 * kq), x1 = ldvec<T, 4>(Ps + i * pld + 16 + 4 * kq);
-        p0 = __builtin_bit_cast(Frag16, x0);
-        p1 = __builtin_bit_cast(Frag16, x1);
+      // V fragments of this wave's column tiles: lane group lg supplies keys 8 lg .. 8 lg + 7 as two transposed reads
+      const T* vrow = Vs + (8 * lg + (li >> 2)) * vld + 4 * (li & 3) + 16 * CT * wv;
+      typename TrRead<T>::v4 lo[CT], hi[CT];
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        if (CT * wv + c < nblk) {
+          lo[c] = TrRead<T>::run(vrow + 16 * c);
+          hi[c] = TrRead<T>::run(vrow + 4 * vld + 16 * c);
+        }
       }
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const int blk = wv + 4 * m;
-        if (blk < nblk) {
-          const int col = blk * 16 + i;
-          Vec<T, 4> v0, v1;
+      for (int rt = 0; rt < 4; ++rt) {
+        if (16 * rt < live_rows) {
+          const Frag pa = *reinterpret_cast<const Frag*>(Ps + (16 * rt + li) * pld + 8 * lg);
 #pragma unroll
-          for (int x = 0; x < 4; ++x) {
-            v0.v[x] = Vs[(4 * kq + x) * vld + col];
-            v1.v[x] = Vs[(16 + 4 * kq + x) * vld + col];
+          for (int c = 0; c < CT; ++c) {
+            if (CT * wv + c < nblk) {
+              typename TrRead<T>::v4 both[2] = {lo[c], hi[c]};
+              acc[rt][c] = Mfma<T>::run(pa, __builtin_bit_cast(Frag, both), acc[rt][c]);
+            }
           }
-          acc[m] = Mfma16<T>::run(p0, __builtin_bit_cast(Frag16, v0), acc[m]);
-          acc[m] = Mfma16<T>::run(p1, __builtin_bit_cast(Frag16, v1), acc[m]);
         }
       }
     }
   }
 #pragma unroll
-  for (int m = 0; m < 4; ++m) {
-    const int blk = wv + 4 * m;
-    if (blk >= nblk) continue;
-    const int c = blk * 16 + (lane & 15);
+  for (int rt = 0; rt < 4; ++rt) {
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int r = 4 * (lane >> 4) + x;
-      const int tl = r / a.heads_per_tile, hl = r - tl * a.heads_per_tile;
-      if (tl >= nt || hl >= nh) continue;
-      if (a.num_splits > 1) {
-        a.partial[(((int64_t)split * a.tokens + t0 + tl) * a.heads + h0 + hl) * dv + c] = acc[m][x];
-      } else {
-        ((T*)a.out)[(t0 + tl) * a.out_token_stride + (int64_t)(h0 + hl) * a.out_head_stride + c] = from_f32<T>(acc[m][x]);
+    for (int c = 0; c < CT; ++c) {
+      if (CT * wv + c >= nblk) continue;
+      const int col = 16 * (CT * wv + c) + li;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int r = 16 * rt + 4 * lg + x;
+        const int tl = r / HR, hl = r - tl * HR;
+        if (tl >= nt || hl >= nh) continue;
+        if (a.num_splits > 1) {
+          a.partial[(((int64_t)split * a.tokens + t0 + tl) * a.heads + h0 + hl) * dv + col] = acc[rt][c][x];
+        } else {
+          ((T*)a.out)[(t0 + tl) * a.out_token_stride + (int64_t)(h0 + hl) * a.out_head_stride + col] = from_f32<T>(acc[rt][c][x]);
+        }
       }
     }
   }
 }
 
+inline bool sg_mfma_shape(int dtype, int d, int dv) {
+  return dtype != MI355_F32 && d % 32 == 0 && dv % 16 == 0 && d <= 32 * SGM_MAXC * 2 && dv <= 32 * SGM_MAXC * 2;
+}
+
 template <typename T> int launch_sigmoid(const SgArgs& a, dim3 grid, bool mfma, hipStream_t stream) {
   if constexpr (!std::is_same<T, float>::value) {
     if (mfma) {
-      const size_t lds = ((size_t)(SG_ROWS + SG_KT) * (a.d + 8) + (size_t)SG_KT * (a.dv + 2) + SG_ROWS * (SG_KT + 8)) * sizeof(T);
-      hipLaunchKernelGGL((sigmoid_attention_mfma_kernel<T>), grid, dim3(256), lds, stream, a);
+      const size_t lds = ((size_t)(SGM_ROWS + SG_KT) * (a.d + 8) + (size_t)SG_KT * (a.dv + 8) + SGM_ROWS * (SG_KT + 8)) * sizeof(T);
+      const int nblk = a.dv / 16;
+#define MI355_SG_LAUNCH(CT)                                                                                                    \
+  do {                                                                                                                         \
+    if (lds > 64 * 1024) {                                                                                                     \
+      hipError_t e = hipFuncSetAttribute((const void*)sigmoid_attention_mfma_kernel<T, CT>,                                    \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                \
+      MI355_REQUIRE(e == hipSuccess, MI355_ERR_LAUNCH, "sigmoid_attention: %zu bytes of LDS refused", lds);                    \
+    }                                                                                                                          \
+    hipLaunchKernelGGL((sigmoid_attention_mfma_kernel<T, CT>), grid, dim3(256), lds, stream, a);                               \
+  } while (0)
+      if (nblk <= 4) MI355_SG_LAUNCH(1);
+      else if (nblk <= 8) MI355_SG_LAUNCH(2);
+      else MI355_SG_LAUNCH(4);
+#undef MI355_SG_LAUNCH
       return MI355_OK;
     }
   }
@@ -306,17 +356,17 @@ template <typename T> int launch_sigmoid(const SgArgs& a, dim3 grid, bool mfma, 
   return MI355_OK;
 }
 
-inline int heads_per_tile(int heads, int kv_heads) { return std::min(heads / kv_heads, SG_ROWS); }
+inline int heads_per_tile(int heads, int kv_heads, int rows) { return std::min(heads / kv_heads, rows); }
 
 }  // namespace
 }  // namespace mi355
 
 using namespace mi355;
 
-int mi355_sigmoid_attention_block_tokens(int heads, int kv_heads, int dtype) {
-  (void)dtype;
+int mi355_sigmoid_attention_block_tokens(int heads, int kv_heads, int head_dim, int v_head_dim, int dtype) {
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads) return 0;
-  return std::max(1, SG_ROWS / heads_per_tile(heads, kv_heads));
+  const int rows = sg_mfma_shape(dtype, head_dim, v_head_dim) ? SGM_ROWS : SG_ROWS;
+  return std::max(1, rows / heads_per_tile(heads, kv_heads, rows));
 }
 
 int mi355_sigmoid_attention(void* out, const void* q, const void* k_cache, const void* v_cache, const int32_t* req_to_token,
@@ -324,7 +374,7 @@ int mi355_sigmoid_attention(void* out, const void* q, const void* k_cache, const
                             const int32_t* blocks, int64_t num_blocks, const float* temp, const float* bias,
                             int64_t q_token_stride, int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride,
                             int64_t req_to_token_stride, int heads, int kv_heads, int head_dim, int v_head_dim, float scale,
-                            int num_splits, float* split_scratch, int64_t tokens, int dtype, void* stream) {
+                            int num_splits, float* split_scratch, int64_t tokens, int max_run, int dtype, void* stream) {
   MI355_REQUIRE(out && q && k_cache && v_cache && req_to_token && req_pool_indices && positions && temp && bias, MI355_ERR_INVALID,
                 "sigmoid_attention: null pointer");
   MI355_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && head_dim > 0 && v_head_dim > 0 && tokens >= 0 &&
@@ -340,14 +390,19 @@ int mi355_sigmoid_attention(void* out, const void* q, const void* k_cache, const
   a.req_pool_indices = req_pool_indices; a.tok_req = tok_req; a.positions = positions; a.blocks = blocks; a.temp = temp;
   a.bias = bias; a.q_token_stride = q_token_stride; a.q_head_stride = q_head_stride; a.out_token_stride = out_token_stride;
   a.out_head_stride = out_head_stride; a.req_to_token_stride = req_to_token_stride; a.tokens = tokens; a.heads = heads;
-  a.kv_heads = kv_heads; a.d = head_dim; a.dv = v_head_dim; a.heads_per_tile = heads_per_tile(heads, kv_heads);
-  a.tokens_per_tile = std::max(1, SG_ROWS / a.heads_per_tile); a.num_splits = num_splits; a.scale = scale;
+  // the matrix-core kernel needs 16-byte rows everywhere; a caller whose q is laid out otherwise gets the vector-ALU kernel,
+  // whose runs are shorter: max_run says how long the caller's runs may be, and a launch that cannot take them is refused
+  const bool mfma = sg_mfma_shape(dtype, head_dim, v_head_dim) && q_token_stride % 8 == 0 && q_head_stride % 8 == 0 &&
+                    aligned16(q) && aligned16(k_cache) && aligned16(v_cache);
+  const int rows = mfma ? SGM_ROWS : SG_ROWS;
+  a.kv_heads = kv_heads; a.d = head_dim; a.dv = v_head_dim; a.heads_per_tile = heads_per_tile(heads, kv_heads, rows);
+  a.tokens_per_tile = std::max(1, rows / a.heads_per_tile); a.num_splits = num_splits; a.scale = scale;
+  MI355_REQUIRE(max_run >= 1 && max_run <= a.tokens_per_tile, MI355_ERR_UNSUPPORTED,
+                "sigmoid_attention: runs of up to %d tokens, this launch takes %d", max_run, a.tokens_per_tile);
   const int rep = heads / kv_heads;
   const int chunks = (rep + a.heads_per_tile - 1) / a.heads_per_tile;
   const dim3 grid((unsigned)num_blocks, (unsigned)(kv_heads * chunks), (unsigned)num_splits);
   MI355_REQUIRE(kv_heads * chunks <= 65535, MI355_ERR_UNSUPPORTED, "sigmoid_attention: too many heads");
-  const bool mfma = dtype != MI355_F32 && head_dim % 32 == 0 && v_head_dim % 16 == 0 && q_token_stride % 8 == 0 &&
-                    q_head_stride % 8 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache);
   int rc = MI355_OK;
   MI355_DISPATCH_DTYPE(dtype, "sigmoid_attention", { rc = launch_sigmoid<T>(a, grid, mfma, (hipStream_t)stream); });
   if (rc != MI355_OK) return rc;

@@ -273,11 +273,142 @@ __global__ __launch_bounds__(256) void moe_grouped_linear_mfma_kernel(T* __restr
     }
 }
 
+
+// Matrix cores through LDS for prefill-sized steps: 128 x 128 output tile (one block of 128 sorted rows of one expert), K in
+// tiles of 64, wave (wm, wn) owns a 64 x 64 quarter as 4 x 4 MFMA 16x16x32 tiles.  The next K tile's rows travel from
+// global memory into registers while the current one is multiplied and are stored to LDS after it; LDS rows are padded by
+// 16 bytes so that the 16-byte fragment reads of 16 consecutive rows fall into different banks.
+constexpr int MOE_WIDE = 128;
+constexpr int MOE_WK = 64;
+constexpr int MOE_WLD = MOE_WK + 8;
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_grouped_linear_wide_kernel(T* __restrict__ out, const T* __restrict__ in,
+                                                                      int64_t in_stride, const T* __restrict__ w,
+                                                                      const int32_t* __restrict__ src_row,
+                                                                      const int32_t* __restrict__ tile_expert,
+                                                                      const int32_t* __restrict__ n_tiles, int gather, int gelu,
+                                                                      int N, int K) {
+  const int tile = blockIdx.y;
+  if (tile >= *n_tiles) return;
+  using Frag = typename Mfma<T>::frag;
+  __shared__ __attribute__((aligned(16))) T As[MOE_WIDE * MOE_WLD];
+  __shared__ __attribute__((aligned(16))) T Bs[MOE_WIDE * MOE_WLD];
+  __shared__ int rowsrc[MOE_WIDE];
+  const int e = tile_expert[tile];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int wm = wv >> 1, wn = wv & 1;
+  const int li = lane & 15, lg = lane >> 4;
+  const int n0 = blockIdx.x * MOE_WIDE;
+  if (tid < MOE_WIDE) {
+    const int sr = src_row[tile * MOE_WIDE + tid];
+    rowsrc[tid] = sr < 0 ? -1 : (gather ? sr : tile * MOE_WIDE + tid);
+  }
+  __syncthreads();
+  const T* we = w + (int64_t)e * N * K;
+  // staging: chunk c = tid + 256 u (u < 4) is row c / 8, 16-byte piece c % 8 of the 64-wide K tile
+  const T* aptr[4];
+  const T* bptr[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int c = tid + 256 * u, r = c >> 3, piece = c & 7;
+    const int sr = rowsrc[r];
+    aptr[u] = sr < 0 ? nullptr : in + (int64_t)sr * in_stride + piece * 8;
+    bptr[u] = (n0 + r < N) ? we + (int64_t)(n0 + r) * K + piece * 8 : nullptr;
+  }
+  Vec<T, 8> zero8;
+#pragma unroll
+  for (int x = 0; x < 8; ++x) zero8.v[x] = from_f32<T>(0.f);
+  Vec<T, 8> areg[4], breg[4];
+  auto request = [&](int k0) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int piece = (tid + 256 * u) & 7;
+      const bool in_k = k0 + piece * 8 < K;
+      areg[u] = (aptr[u] != nullptr && in_k) ? ldvec<T, 8>(aptr[u] + k0) : zero8;
+      breg[u] = (bptr[u] != nullptr && in_k) ? ldvec<T, 8>(bptr[u] + k0) : zero8;
+    }
+  };
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int y = 0; y < 4; ++y) acc[x][y] = f32x4{0.f, 0.f, 0.f, 0.f};
+  request(0);
+  for (int k0 = 0; k0 < K; k0 += MOE_WK) {
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = tid + 256 * u, r = c >> 3, piece = c & 7;
+      stvec<T, 8>(As + r * MOE_WLD + piece * 8, areg[u]);
+      stvec<T, 8>(Bs + r * MOE_WLD + piece * 8, breg[u]);
+    }
+    __syncthreads();
+    if (k0 + MOE_WK < K) request(k0 + MOE_WK);
+#pragma unroll
+    for (int kk = 0; kk < MOE_WK; kk += 32) {
+      Frag af[4], bf[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        af[x] = *reinterpret_cast<const Frag*>(As + (wm * 64 + x * 16 + li) * MOE_WLD + kk + 8 * lg);
+        bf[x] = *reinterpret_cast<const Frag*>(Bs + (wn * 64 + x * 16 + li) * MOE_WLD + kk + 8 * lg);
+      }
+#pragma unroll
+      for (int x = 0; x < 4; ++x)
+#pragma unroll
+        for (int y = 0; y < 4; ++y) acc[x][y] = Mfma<T>::run(af[x], bf[y], acc[x][y]);
+    }
+  }
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = wm * 64 + x * 16 + 4 * lg + r;
+      const bool live = rowsrc[row] >= 0;
+      T* dst = out + (int64_t)(tile * MOE_WIDE + row) * N;
+#pragma unroll
+      for (int y = 0; y < 4; ++y) {
+        const int n = n0 + wn * 64 + y * 16 + li;
+        if (n >= N) continue;
+        float v = live ? acc[x][y][r] : 0.f;
+        if (gelu) v = moe_gelu_erf(v);
+        dst[n] = from_f32<T>(v);
+      }
+    }
+}
+
+// Exact fp32 logits of few rows against a small table: out[t][n] = x[t] . w[n].  One wave per row, the row staged in LDS
+// once and read against every table row; meant for decode-sized steps, where a tiled GEMM would occupy a handful of CUs.
+__global__ __launch_bounds__(256) void moe_router_logits_kernel(float* __restrict__ out, const float* __restrict__ x,
+                                                                const float* __restrict__ w, int64_t rows, int N, int K) {
+  extern __shared__ __attribute__((aligned(16))) float smx[];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int64_t t = (int64_t)blockIdx.x * 4 + wv;
+  float* xr = smx + (int64_t)wv * K;
+  if (t < rows)
+    for (int k = lane; k < K; k += 64) xr[k] = x[t * K + k];
+  __syncthreads();
+  if (t >= rows) return;
+  for (int n = 0; n < N; ++n) {
+    const float* wr = w + (int64_t)n * K;
+    float acc = 0.f;
+    for (int k = lane; k < K; k += 64) acc = fmaf(xr[k], wr[k], acc);
+    acc = wave_sum(acc);
+    if (lane == 0) out[t * N + n] = acc;
+  }
+}
+
 template <typename T>
 int launch_grouped(void* out, const void* in, int64_t in_stride, const void* w, const int32_t* src_row, const int32_t* tile_expert,
-                   const int32_t* n_tiles, int gather, int gelu, int N, int K, int64_t max_tiles, bool mfma, hipStream_t stream) {
-  const dim3 grid((unsigned)cdiv(N, 64), (unsigned)max_tiles);
+                   const int32_t* n_tiles, int gather, int gelu, int N, int K, int64_t max_tiles, bool mfma, int block,
+                   hipStream_t stream) {
+  const dim3 grid((unsigned)cdiv(N, block), (unsigned)max_tiles);
   if constexpr (!std::is_same<T, float>::value) {
+    if (mfma && block == MOE_WIDE) {
+      hipLaunchKernelGGL((moe_grouped_linear_wide_kernel<T>), grid, dim3(256), 0, stream, (T*)out, (const T*)in, in_stride,
+                         (const T*)w, src_row, tile_expert, n_tiles, gather, gelu, N, K);
+      return MI355_OK;
+    }
     if (mfma) {
       hipLaunchKernelGGL((moe_grouped_linear_mfma_kernel<T>), grid, dim3(256), 0, stream, (T*)out, (const T*)in, in_stride,
                          (const T*)w, src_row, tile_expert, n_tiles, gather, gelu, N, K);
@@ -309,34 +440,49 @@ int mi355_moe_route_grouped(int32_t* ids, float* weights, const float* logits, c
   return MI355_OK;
 }
 
-int mi355_moe_block_rows(void) { return MOE_BLOCK; }
+int mi355_moe_block_rows(int wide) { return wide ? MOE_WIDE : MOE_BLOCK; }
+
+int mi355_moe_router_logits(float* out, const float* x, const float* weight, int64_t rows, int n, int k, void* stream) {
+  MI355_REQUIRE(out && x && weight, MI355_ERR_INVALID, "moe_router_logits: null pointer");
+  MI355_REQUIRE(rows >= 0 && n > 0 && k > 0 && k <= 8192, MI355_ERR_INVALID, "moe_router_logits: bad shape");
+  if (rows == 0) return MI355_OK;
+  hipLaunchKernelGGL(moe_router_logits_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), (size_t)4 * k * sizeof(float),
+                     (hipStream_t)stream, out, x, weight, rows, n, k);
+  MI355_CHECK_LAUNCH("moe_router_logits");
+  return MI355_OK;
+}
 
 int mi355_moe_align(int32_t* src_row, int32_t* rows, int32_t* tile_expert, int32_t* n_tiles, const int32_t* ids, int64_t tokens,
-                    int top, int num_experts, int64_t padded, void* stream) {
+                    int top, int num_experts, int block, int64_t padded, void* stream) {
+  MI355_REQUIRE(block == MOE_BLOCK || block == MOE_WIDE, MI355_ERR_INVALID, "moe_align: blocks of %d or %d rows", MOE_BLOCK, MOE_WIDE);
   MI355_REQUIRE(src_row && rows && tile_expert && n_tiles && ids, MI355_ERR_INVALID, "moe_align: null pointer");
   MI355_REQUIRE(tokens >= 0 && top > 0 && num_experts > 0 && num_experts <= 4096, MI355_ERR_INVALID, "moe_align: bad shape");
-  MI355_REQUIRE(padded % MOE_BLOCK == 0 && padded >= tokens * top + (int64_t)std::min<int64_t>(num_experts, tokens * top) * (MOE_BLOCK - 1),
+  MI355_REQUIRE(padded % block == 0 && padded >= tokens * top + (int64_t)std::min<int64_t>(num_experts, tokens * top) * (block - 1),
                 MI355_ERR_INVALID, "moe_align: %lld padded rows cannot hold %lld pairs of %d experts", (long long)padded,
                 (long long)(tokens * top), num_experts);
   const size_t lds = (size_t)(2 * num_experts + 1) * sizeof(int);
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), lds, (hipStream_t)stream, src_row, rows, tile_expert, n_tiles, ids,
-                     tokens * top, top, num_experts, MOE_BLOCK, padded);
+                     tokens * top, top, num_experts, block, padded);
   MI355_CHECK_LAUNCH("moe_align");
   return MI355_OK;
 }
 
 int mi355_moe_grouped_linear(void* out, const void* in, int64_t in_stride, const void* weight, const int32_t* src_row,
-                             const int32_t* tile_expert, const int32_t* n_tiles, int gather, int gelu, int64_t padded, int n, int k,
-                             int dtype, void* stream) {
+                             const int32_t* tile_expert, const int32_t* n_tiles, int gather, int gelu, int64_t padded, int block,
+                             int n, int k, int dtype, void* stream) {
   MI355_REQUIRE(out && in && weight && src_row && tile_expert && n_tiles, MI355_ERR_INVALID, "moe_grouped_linear: null pointer");
-  MI355_REQUIRE(padded >= 0 && padded % MOE_BLOCK == 0 && n > 0 && k > 0 && in_stride >= k && padded / MOE_BLOCK <= 65535,
+  MI355_REQUIRE(block == MOE_BLOCK || block == MOE_WIDE, MI355_ERR_INVALID, "moe_grouped_linear: blocks of %d or %d rows", MOE_BLOCK,
+                MOE_WIDE);
+  MI355_REQUIRE(padded >= 0 && padded % block == 0 && n > 0 && k > 0 && in_stride >= k && padded / block <= 65535,
                 MI355_ERR_INVALID, "moe_grouped_linear: bad shape");
   if (padded == 0) return MI355_OK;
   const bool mfma = dtype != MI355_F32 && k % 8 == 0 && in_stride % 8 == 0 && aligned16(in) && aligned16(weight);
+  MI355_REQUIRE(block == MOE_BLOCK || mfma, MI355_ERR_UNSUPPORTED,
+                "moe_grouped_linear: blocks of %d rows are for 16-bit operands with 16-byte rows", MOE_WIDE);
   int rc = MI355_OK;
   MI355_DISPATCH_DTYPE(dtype, "moe_grouped_linear", {
-    rc = launch_grouped<T>(out, in, in_stride, weight, src_row, tile_expert, n_tiles, gather, gelu, n, k, padded / MOE_BLOCK, mfma,
-                           (hipStream_t)stream);
+    rc = launch_grouped<T>(out, in, in_stride, weight, src_row, tile_expert, n_tiles, gather, gelu, n, k, padded / block, mfma,
+                           block, (hipStream_t)stream);
   });
   if (rc != MI355_OK) return rc;
   MI355_CHECK_LAUNCH("moe_grouped_linear");

@@ -322,7 +322,7 @@ class Mi355AttnBackend(AttentionBackend):
         ranges whose partial sums a second launch adds (the weights are not normalised, so partial sums simply add)."""
         ops = get_ops()
         k_cache, v_cache = forward_batch.token_to_kv_pool.get_kv_buffer(layer.layer_id)
-        bq = ops.sigmoid_attention_block_tokens(layer.tp_q_head_num, layer.tp_k_head_num, q.dtype)
+        bq = ops.sigmoid_attention_block_tokens(layer.tp_q_head_num, layer.tp_k_head_num, layer.qk_head_dim, layer.v_head_dim, q.dtype)
         splits = 1
         if forward_batch.forward_mode.is_decode() and forward_batch.seq_lens_cpu is not None:
             splits = ops.sigmoid_attention_splits(q.shape[0], layer.tp_q_head_num, layer.tp_k_head_num,
@@ -330,7 +330,7 @@ class Mi355AttnBackend(AttentionBackend):
         return ops.sigmoid_attention(
             q, k_cache, v_cache, out, forward_batch.req_to_token_pool.req_to_token, forward_batch.req_pool_indices,
             forward_batch.positions, layer.temp.data, layer.bias.data, layer.scaling,
-            tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq), num_splits=splits)
+            tok_req=forward_batch.token_req_index(), blocks=self._latent_blocks(forward_batch, bq), num_splits=splits, max_run=bq)
 
     def _windowed(self, layer) -> bool:
         """triton_backend.py:656, 711: a layer with sliding_window_size > -1 attends the window lists."""

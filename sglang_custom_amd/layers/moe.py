@@ -31,7 +31,7 @@ class GroupedTopKRouter(nn.Module):
     def forward(self, x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
         """x fp32 [T, D] -> (expert ids int32 [T, top], weights fp32 [T, top])."""
         ops = get_ops()
-        logits = ops.linear(x, self.weight.data)
+        logits = ops.moe_router_logits(x, self.weight.data)
         return ops.moe_route_grouped(logits, self.correction.data, self.top, self.n_groups, self.keep_groups, self.scale)
 
 
@@ -47,7 +47,8 @@ class GroupedExperts(nn.Module):
         """h [T, D], expert_ids int32 [T, top] -> (y [P, D], rows int32 [T, top]): y[rows[t, j]] is the output of token
         t's j-th expert; P >= T * top counts the padding of the experts' blocks."""
         ops = get_ops()
-        plan = ops.moe_align(expert_ids, self.num_experts)
+        plan = ops.moe_align(expert_ids, self.num_experts,
+                             wide_ok=h.dtype != torch.float32 and self.hidden % 8 == 0 and self.ff % 8 == 0)
         a = ops.moe_grouped_linear(h, self.w_up.data, plan, gather=True, gelu=True)
         y = ops.moe_grouped_linear(a, self.w_down.data, plan, gather=False, gelu=False)
         return y, plan.rows

@@ -1379,22 +1379,23 @@ def linear_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: to
 
 
 # ------------------------------------------------------- causal attention with sigmoid weights
-def sigmoid_attention_block_tokens(heads: int, kv_heads: int, dtype: torch.dtype) -> int:
+def sigmoid_attention_block_tokens(heads: int, kv_heads: int, head_dim: int, v_head_dim: int, dtype: torch.dtype) -> int:
     """Most consecutive tokens of one sequence that a workgroup of sigmoid_attention takes."""
-    return int(_lib_().mi355_sigmoid_attention_block_tokens(heads, kv_heads, _DT[dtype]))
+    return int(_lib_().mi355_sigmoid_attention_block_tokens(heads, kv_heads, head_dim, v_head_dim, _DT[dtype]))
 
 
 def sigmoid_attention_splits(tokens: int, heads: int, kv_heads: int, max_len: int, dtype: torch.dtype) -> int:
-    """Key ranges per token for a decode-sized launch: enough workgroups to cover the chip twice, at least 128 keys each."""
-    wgs = max(1, tokens * kv_heads * ((heads // kv_heads + 15) // 16))
-    return int(max(1, min(64, (512 + wgs - 1) // wgs, max_len // 128)))
+    """Key ranges per token for a decode-sized launch: eight workgroups per CU in flight (a workgroup waits on its own
+    loads; its neighbours' products cover them), at least 128 keys each."""
+    wgs = max(1, tokens * kv_heads * ((heads // kv_heads + 63) // 64))
+    return int(max(1, min(64, (2048 + wgs - 1) // wgs, max_len // 128)))
 
 
 def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, req_to_token: torch.Tensor,
                       req_pool_indices: torch.Tensor, positions: torch.Tensor, temp: torch.Tensor, bias: torch.Tensor, scale: float,
-                      tok_req=None, blocks=None, num_splits: int = 1) -> torch.Tensor:
+                      tok_req=None, blocks=None, num_splits: int = 1, max_run: Optional[int] = None) -> torch.Tensor:
     """q [T, H, d], caches [slots, G, d] / [slots, G, dv], out [T, H, dv]; temp / bias fp32 [H]; blocks int32 [n, 2] runs of
-    consecutive tokens of one sequence or None (one token per run)."""
+    at most max_run consecutive tokens of one sequence, or None (one token per run)."""
     _gpu(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, temp, bias, tok_req, blocks)
     T, H, d = q.shape
     G, dv = k_cache.shape[1], v_cache.shape[2]
@@ -1407,14 +1408,15 @@ def sigmoid_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     if blocks is not None:
         assert blocks.dtype == torch.int32 and blocks.dim() == 2 and blocks.shape[1] == 2 and blocks.is_contiguous()
         nb, num_splits = blocks.shape[0], 1
+        assert max_run is not None, "runs come with their longest length"
     else:
-        nb = T
+        nb, max_run = T, 1
     scratch = torch.empty(num_splits * T * H * dv, dtype=torch.float32, device=q.device) if num_splits > 1 else None
     check(_lib_().mi355_sigmoid_attention(
         out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), req_to_token.data_ptr(), req_pool_indices.data_ptr(),
         _p(tok_req), positions.data_ptr(), _p(blocks), nb, temp.data_ptr(), bias.data_ptr(), q.stride(0), q.stride(1),
-        out.stride(0), out.stride(1), req_to_token.stride(0), H, G, d, dv, float(scale), int(num_splits), _p(scratch), T, _dt(q),
-        _stream(q)), "sigmoid_attention")
+        out.stride(0), out.stride(1), req_to_token.stride(0), H, G, d, dv, float(scale), int(num_splits), _p(scratch), T,
+        int(max_run), _dt(q), _stream(q)), "sigmoid_attention")
     return out
 
 
@@ -1441,11 +1443,31 @@ class MoePlan:
         self.src_row, self.rows, self.tile_expert, self.n_tiles, self.block, self.padded = src_row, rows, tile_expert, n_tiles, block, padded
 
 
-def moe_align(expert_ids: torch.Tensor, num_experts: int) -> MoePlan:
+ROUTER_SKINNY_MAX_ROWS = 256
+
+
+def moe_router_logits(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """fp32 x [T, D] against the fp32 router table [E, D] -> exact fp32 logits [T, E].  Few rows go to a wave-per-row kernel
+    (a tiled GEMM with E columns would occupy a handful of CUs), many to the exact tiled GEMM."""
+    _gpu(x, weight)
+    assert x.dtype == torch.float32 and weight.dtype == torch.float32 and x.is_contiguous() and weight.is_contiguous()
+    T, K = x.shape
+    if T > ROUTER_SKINNY_MAX_ROWS or K > 8192:
+        return linear(x, weight)
+    out = torch.empty((T, weight.shape[0]), dtype=torch.float32, device=x.device)
+    check(_lib_().mi355_moe_router_logits(out.data_ptr(), x.data_ptr(), weight.data_ptr(), T, weight.shape[0], K, _stream(x)),
+          "moe_router_logits")
+    return out
+
+
+def moe_align(expert_ids: torch.Tensor, num_experts: int, wide_ok: bool = False) -> MoePlan:
+    """wide_ok: the grouped GEMMs that follow can take blocks of 128 rows (16-bit operands, 16-byte rows); they are used
+    when the experts have at least two such blocks' worth of rows on average."""
     _gpu(expert_ids)
     T, top = expert_ids.shape
     assert expert_ids.dtype == torch.int32 and expert_ids.is_contiguous()
-    block = int(_lib_().mi355_moe_block_rows())
+    wide = bool(wide_ok) and T * top >= 256 * num_experts
+    block = int(_lib_().mi355_moe_block_rows(int(wide)))
     pairs = T * top
     padded = (pairs + min(num_experts, pairs) * (block - 1) + block - 1) // block * block
     dev = expert_ids.device
@@ -1454,7 +1476,7 @@ def moe_align(expert_ids: torch.Tensor, num_experts: int) -> MoePlan:
     tile_expert = torch.empty(max(padded // block, 1), dtype=torch.int32, device=dev)
     n_tiles = torch.empty(1, dtype=torch.int32, device=dev)
     check(_lib_().mi355_moe_align(src_row.data_ptr(), rows.data_ptr(), tile_expert.data_ptr(), n_tiles.data_ptr(),
-                                  expert_ids.data_ptr(), T, top, int(num_experts), padded, _stream(expert_ids)), "moe_align")
+                                  expert_ids.data_ptr(), T, top, int(num_experts), block, padded, _stream(expert_ids)), "moe_align")
     return MoePlan(src_row, rows, tile_expert, n_tiles, block, padded)
 
 
@@ -1468,5 +1490,5 @@ def moe_grouped_linear(x: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: 
     out = torch.empty((plan.padded, N), dtype=x.dtype, device=x.device)
     check(_lib_().mi355_moe_grouped_linear(out.data_ptr(), x.data_ptr(), x.stride(0), w.data_ptr(), plan.src_row.data_ptr(),
                                            plan.tile_expert.data_ptr(), plan.n_tiles.data_ptr(), int(gather), int(gelu),
-                                           plan.padded, N, K, _dt(x), _stream(x)), "moe_grouped_linear")
+                                           plan.padded, plan.block, N, K, _dt(x), _stream(x)), "moe_grouped_linear")
     return out

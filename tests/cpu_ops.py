@@ -409,7 +409,7 @@ def head_rmsnorm_gate(o, weight, gate, eps, out_dtype):
     return (n * g * torch.sigmoid(g)).reshape(T, H * dv).to(out_dtype)
 
 
-def sigmoid_attention_block_tokens(heads, kv_heads, dtype):
+def sigmoid_attention_block_tokens(heads, kv_heads, head_dim, v_head_dim, dtype):
     return 3
 
 
@@ -418,7 +418,7 @@ def sigmoid_attention_splits(tokens, heads, kv_heads, max_len, dtype):
 
 
 def sigmoid_attention(q, k_cache, v_cache, out, req_to_token, req_pool_indices, positions, temp, bias, scale, tok_req=None,
-                      blocks=None, num_splits=1):
+                      blocks=None, num_splits=1, max_run=None):
     T, H, d = q.shape
     G = k_cache.shape[1]
     covered = torch.zeros(T, dtype=torch.bool)
@@ -456,7 +456,11 @@ def moe_route_grouped(logits, correction, top, n_groups, keep_groups, scale):
     return ids, w
 
 
-def moe_align(expert_ids, num_experts, block=4):
+def moe_router_logits(x, weight):
+    return F.linear(x, weight)
+
+
+def moe_align(expert_ids, num_experts, wide_ok=False, block=4):
     T, top = expert_ids.shape
     flat = expert_ids.reshape(-1).tolist()
     src, tiles = [], []

@@ -212,3 +212,4 @@ def test_standins_recurrence_attention_mixture():
     cases.check_router(cpu_ops, "cpu")
     cases.check_router(cpu_ops, "cpu", E=8, n_groups=8, keep=3, top=2)
     cases.check_experts(cpu_ops, "cpu", torch.float32)
+    cases.check_router_logits(cpu_ops, "cpu", 5)

@@ -98,6 +98,18 @@ def test_experts_over_sorted_blocks(dtype, T, D, ff, E, top):
     cases.check_experts(ops(), DEV, dtype, T=T, D=D, ff=ff, E=E, top=top)
 
 
+@pytest.mark.parametrize("D,ff", [(64, 96), (200, 72), (256, 128)])
+def test_experts_over_wide_blocks(D, ff):
+    """Enough rows per expert for the 128-row blocks of the prefill-sized kernel: K tiles with a tail (200, 72), one idle
+    expert, column counts that are no multiple of the tile."""
+    cases.check_experts(ops(), DEV, torch.bfloat16, T=1100, D=D, ff=ff, E=4, top=2, wide_ok=True)
+
+
+def test_router_logits_few_rows_and_many():
+    for T in (1, 5, 64, 300):
+        cases.check_router_logits(ops(), DEV, T)
+
+
 # ---------------------------------------------------------------------------------------------- the engine
 CASES = [("float32", 3e-5), ("bfloat16", 6e-2)]
 

@@ -209,7 +209,7 @@ def run_sigmoid_attention(ops, device, dtype, q, kn, v, scale, temp, bias, cuts,
     T, H, d = q.shape
     G = kn.shape[1]
     kv = KVSetup(device, dtype, kn, v, page=page)
-    bq = ops.sigmoid_attention_block_tokens(H, G, dtype)
+    bq = ops.sigmoid_attention_block_tokens(H, G, d, v.shape[-1], dtype)
     qd = q.to(dtype).to(device)
     outs, at = [], 0
     for n in cuts:
@@ -222,7 +222,7 @@ def run_sigmoid_attention(ops, device, dtype, q, kn, v, scale, temp, bias, cuts,
             blocks = torch.tensor(runs, dtype=torch.int32, device=device)
         ops.sigmoid_attention(qd[at:at + n], kv.k_cache, kv.v_cache, o, kv.tab.req_to_token, b["req_pool_indices"], b["positions"],
                               temp.float().to(device), bias.float().to(device), scale, tok_req=None if decode else b["tok_req"],
-                              blocks=blocks, num_splits=splits if decode else 1)
+                              blocks=blocks, num_splits=splits if decode else 1, max_run=bq)
         outs.append(o.cpu())
         at += n
     return torch.cat(outs)
@@ -292,7 +292,13 @@ def check_router(ops, device, E=12, n_groups=4, keep=2, top=3, scale=1.5, T=64):
         assert abs(float(wt[t].sum()) - scale) < 1e-5
 
 
-def check_experts(ops, device, dtype, T=37, D=48, ff=40, E=5, top=2):
+def check_router_logits(ops, device, T, D=200, E=12):
+    g = torch.Generator().manual_seed(9)
+    x, w = torch.randn(T, D, generator=g), torch.randn(E, D, generator=g)
+    _close(ops.moe_router_logits(x.to(device), w.to(device)), x.double() @ w.double().T, 2e-6, "router logits in fp32")
+
+
+def check_experts(ops, device, dtype, T=37, D=48, ff=40, E=5, top=2, wide_ok=False):
     g = torch.Generator().manual_seed(6)
     h = _bf(torch.randn(T, D, generator=g))
     up = _bf(torch.randn(E, ff, D, generator=g) * D ** -0.5)
@@ -303,7 +309,7 @@ def check_experts(ops, device, dtype, T=37, D=48, ff=40, E=5, top=2):
         for t in range(T):
             if -1 in ids[t].tolist():
                 ids[t][ids[t] == -1] = [e for e in range(E - 1) if e not in ids[t].tolist()][0]
-    plan = ops.moe_align(ids.to(device), E)
+    plan = ops.moe_align(ids.to(device), E, wide_ok=wide_ok)
     a = ops.moe_grouped_linear(h.to(dtype).to(device), up.to(dtype).to(device), plan, gather=True, gelu=True)
     y = ops.moe_grouped_linear(a, down.to(dtype).to(device), plan, gather=False, gelu=False)
     rows = plan.rows.cpu().long()
