@@ -220,21 +220,17 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
   const T* vc = (const T*)a.v_cache;
   using Frag = typename Mfma<T>::frag;
   Vec<T, 8> kreg[SGM_MAXC], vreg[SGM_MAXC];
+  // every load is unconditional (a load under a branch is waited for at the branch's end, one latency per load): chunk
+  // numbers past the tile's last one are clamped to it -- all lanes then read one address -- and never stored
   auto request = [&](int tile) {
     const int j0 = tile * SG_KT;
 #pragma unroll
     for (int u = 0; u < SGM_MAXC; ++u) {
-      const int e = tid + 256 * u;
-      if (e < SG_KT * dch) {
-        const int kk = e / dch, ch = e - kk * dch;
-        const int j = min(j0 + kk, last);        // keys past the run's last one are masked below; any valid row will do
-        kreg[u] = ldvec<T, 8>(kc + ((int64_t)table[j] * a.kv_heads + g) * d + ch * 8);
-      }
-      if (e < SG_KT * vch) {
-        const int kk = e / vch, ch = e - kk * vch;
-        const int j = min(j0 + kk, last);
-        vreg[u] = ldvec<T, 8>(vc + ((int64_t)table[j] * a.kv_heads + g) * dv + ch * 8);
-      }
+      const int ek = min(tid + 256 * u, SG_KT * dch - 1), ev = min(tid + 256 * u, SG_KT * vch - 1);
+      const int kk = ek / dch, kv = ev / vch;
+      // keys past the run's last one are masked below; any valid row will do
+      kreg[u] = ldvec<T, 8>(kc + ((int64_t)table[min(j0 + kk, last)] * a.kv_heads + g) * d + (ek - kk * dch) * 8);
+      vreg[u] = ldvec<T, 8>(vc + ((int64_t)table[min(j0 + kv, last)] * a.kv_heads + g) * dv + (ev - kv * vch) * 8);
     }
   };
   if (tile_lo < tile_hi) request(tile_lo);

@@ -228,15 +228,17 @@ __global__ __launch_bounds__(256) void moe_grouped_linear_mfma_kernel(T* __restr
   const int n0 = blockIdx.x * 64 + wn * 32;
   const int i = lane & 15, kq = lane >> 4;
   const T* we = w + (int64_t)e * N * K;
+  // every load is unconditional: padding rows and columns past N read row 0 (their products are never stored), the K
+  // tail is zeroed by a select
   const T* arow[2];
   const T* brow[2];
 #pragma unroll
   for (int x = 0; x < 2; ++x) {
     const int p = tile * MOE_BLOCK + wm * 32 + x * 16 + i;
     const int s = src_row[p];
-    arow[x] = s < 0 ? nullptr : in + (int64_t)(gather ? s : p) * in_stride;
+    arow[x] = in + (int64_t)(s < 0 ? 0 : (gather ? s : p)) * in_stride;
     const int n = n0 + x * 16 + i;
-    brow[x] = n < N ? we + (int64_t)n * K : nullptr;
+    brow[x] = we + (int64_t)(n < N ? n : 0) * K;
   }
   f32x4 acc[2][2];
 #pragma unroll
@@ -245,12 +247,14 @@ __global__ __launch_bounds__(256) void moe_grouped_linear_mfma_kernel(T* __restr
     for (int y = 0; y < 2; ++y) acc[x][y] = f32x4{0.f, 0.f, 0.f, 0.f};
   const Frag zero = {};
   for (int k0 = 0; k0 < K; k0 += 32) {
-    const int k = k0 + 8 * kq;
+    const bool in_k = k0 + 8 * kq < K;
+    const int k = in_k ? k0 + 8 * kq : 0;
     Frag af[2], bf[2];
 #pragma unroll
     for (int x = 0; x < 2; ++x) {
-      af[x] = (arow[x] != nullptr && k < K) ? *reinterpret_cast<const Frag*>(arow[x] + k) : zero;
-      bf[x] = (brow[x] != nullptr && k < K) ? *reinterpret_cast<const Frag*>(brow[x] + k) : zero;
+      const Frag av = *reinterpret_cast<const Frag*>(arow[x] + k);
+      af[x] = in_k ? av : zero;
+      bf[x] = *reinterpret_cast<const Frag*>(brow[x] + k);
     }
 #pragma unroll
     for (int x = 0; x < 2; ++x)
@@ -278,6 +282,12 @@ __global__ __launch_bounds__(256) void moe_grouped_linear_mfma_kernel(T* __restr
 // tiles of 64, wave (wm, wn) owns a 64 x 64 quarter as 4 x 4 MFMA 16x16x32 tiles.  The next K tile's rows travel from
 // global memory into registers while the current one is multiplied and are stored to LDS after it; LDS rows are padded by
 // 16 bytes so that the 16-byte fragment reads of 16 consecutive rows fall into different banks.
+// one 16-byte load, spelled as a vector of four dwords so that it cannot be taken apart
+typedef unsigned moe_u32x4 __attribute__((ext_vector_type(4)));
+template <typename T> __device__ __forceinline__ Vec<T, 8> ld16(const T* p) {
+  return __builtin_bit_cast(Vec<T, 8>, *reinterpret_cast<const moe_u32x4*>(p));
+}
+
 constexpr int MOE_WIDE = 128;
 constexpr int MOE_WK = 64;
 constexpr int MOE_WLD = MOE_WK + 8;
@@ -306,27 +316,32 @@ __global__ __launch_bounds__(256) void moe_grouped_linear_wide_kernel(T* __restr
   }
   __syncthreads();
   const T* we = w + (int64_t)e * N * K;
-  // staging: chunk c = tid + 256 u (u < 4) is row c / 8, 16-byte piece c % 8 of the 64-wide K tile
+  // staging: chunk c = tid + 256 u (u < 4) is row c / 8, 16-byte piece c % 8 of the 64-wide K tile.  Every load is
+  // unconditional (a load under a branch is waited for at the branch's end, one latency per load): padding rows and
+  // columns past N read row 0 -- their products are never stored -- and only the K tail is zeroed, by a select.
   const T* aptr[4];
   const T* bptr[4];
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     const int c = tid + 256 * u, r = c >> 3, piece = c & 7;
     const int sr = rowsrc[r];
-    aptr[u] = sr < 0 ? nullptr : in + (int64_t)sr * in_stride + piece * 8;
-    bptr[u] = (n0 + r < N) ? we + (int64_t)(n0 + r) * K + piece * 8 : nullptr;
+    aptr[u] = in + (int64_t)(sr < 0 ? 0 : sr) * in_stride + piece * 8;
+    bptr[u] = we + (int64_t)(n0 + r < N ? n0 + r : 0) * K + piece * 8;
   }
   Vec<T, 8> zero8;
 #pragma unroll
   for (int x = 0; x < 8; ++x) zero8.v[x] = from_f32<T>(0.f);
   Vec<T, 8> areg[4], breg[4];
+  const bool k_tail = K % MOE_WK != 0;
   auto request = [&](int k0) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int piece = (tid + 256 * u) & 7;
-      const bool in_k = k0 + piece * 8 < K;
-      areg[u] = (aptr[u] != nullptr && in_k) ? ldvec<T, 8>(aptr[u] + k0) : zero8;
-      breg[u] = (bptr[u] != nullptr && in_k) ? ldvec<T, 8>(bptr[u] + k0) : zero8;
+      const bool in_k = !k_tail || k0 + piece * 8 < K;
+      const int kk = in_k ? k0 : 0;
+      const Vec<T, 8> av = ld16<T>(aptr[u] + kk), bv = ld16<T>(bptr[u] + kk);
+      areg[u] = in_k ? av : zero8;
+      breg[u] = bv;
     }
   };
   f32x4 acc[4][4];
