@@ -765,7 +765,7 @@ int mi355_sigmoid_attention(void* out, const void* q, const void* k_cache, const
  *   n_groups equal groups of neighbours, a group scores the sum of its two largest selection scores (its only one, for
  *   groups of one), the keep_groups best groups stay, the `top` largest selection scores among them are chosen (ties: the
  *   smaller index); weights[t][k] = s[chosen] / (sum of the chosen s + 1e-20) * scale.
- * mi355_moe_router_logits: out[t][j] = x[t] . weight[j] in exact fp32 for few rows (one wave per row; k <= 8192).
+ * mi355_moe_router_logits: out[t][j] = x[t] . weight[j] in exact fp32 for few rows (one workgroup per row; k <= 16384).
  * mi355_moe_align: sorts the tokens * top (token, choice) pairs by expert into blocks of `block` rows
  *   (mi355_moe_block_rows(0), or mi355_moe_block_rows(1) for prefill-sized steps of 16-bit models) of one expert each: src_row[p] = token of sorted row p or -1 (padding), rows[pair] = p, tile_expert[block] = its expert,
  *   *n_tiles = blocks in use.  `padded` (a multiple of the block) must be at least pairs + min(experts, pairs) * (block - 1).

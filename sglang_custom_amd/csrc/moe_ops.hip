@@ -392,24 +392,40 @@ __global__ __launch_bounds__(256) void moe_grouped_linear_wide_kernel(T* __restr
     }
 }
 
-// Exact fp32 logits of few rows against a small table: out[t][n] = x[t] . w[n].  One wave per row, the row staged in LDS
-// once and read against every table row; meant for decode-sized steps, where a tiled GEMM would occupy a handful of CUs.
+// Exact fp32 logits of few rows against a small table: out[t][n] = x[t] . w[n].  One workgroup per row: the row is staged
+// in LDS once, wave v takes table rows v, v + 4, ..., four at a time so that sixteen loads are in flight per lane; meant for
+// decode-sized steps, where a tiled GEMM with so few columns would occupy a handful of CUs.
 __global__ __launch_bounds__(256) void moe_router_logits_kernel(float* __restrict__ out, const float* __restrict__ x,
-                                                                const float* __restrict__ w, int64_t rows, int N, int K) {
+                                                                const float* __restrict__ w, int N, int K) {
   extern __shared__ __attribute__((aligned(16))) float smx[];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int64_t t = (int64_t)blockIdx.x * 4 + wv;
-  float* xr = smx + (int64_t)wv * K;
-  if (t < rows)
-    for (int k = lane; k < K; k += 64) xr[k] = x[t * K + k];
+  const int64_t t = blockIdx.x;
+  for (int k = threadIdx.x; k < K; k += 256) smx[k] = x[t * K + k];
   __syncthreads();
-  if (t >= rows) return;
-  for (int n = 0; n < N; ++n) {
-    const float* wr = w + (int64_t)n * K;
-    float acc = 0.f;
-    for (int k = lane; k < K; k += 64) acc = fmaf(xr[k], wr[k], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) out[t * N + n] = acc;
+  const bool vec = (K & 3) == 0 && aligned16(w);
+  for (int nb = wv; nb < N; nb += 16) {        // this wave's rows nb, nb + 4, nb + 8, nb + 12
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (vec) {
+      for (int k = 4 * lane; k < K; k += 256) {
+        const float4 xv = *reinterpret_cast<const float4*>(smx + k);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int n = min(nb + 4 * j, N - 1);   // rows past the table read its last row; their sums are dropped
+          const float4 wv4 = *reinterpret_cast<const float4*>(w + (int64_t)n * K + k);
+          acc[j] = fmaf(xv.x, wv4.x, fmaf(xv.y, wv4.y, fmaf(xv.z, wv4.z, fmaf(xv.w, wv4.w, acc[j]))));
+        }
+      }
+    } else {
+      for (int k = lane; k < K; k += 64) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = fmaf(smx[k], w[(int64_t)min(nb + 4 * j, N - 1) * K + k], acc[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float sum = wave_sum(acc[j]);
+      if (lane == 0 && nb + 4 * j < N) out[t * N + nb + 4 * j] = sum;
+    }
   }
 }
 
@@ -459,10 +475,10 @@ int mi355_moe_block_rows(int wide) { return wide ? MOE_WIDE : MOE_BLOCK; }
 
 int mi355_moe_router_logits(float* out, const float* x, const float* weight, int64_t rows, int n, int k, void* stream) {
   MI355_REQUIRE(out && x && weight, MI355_ERR_INVALID, "moe_router_logits: null pointer");
-  MI355_REQUIRE(rows >= 0 && n > 0 && k > 0 && k <= 8192, MI355_ERR_INVALID, "moe_router_logits: bad shape");
+  MI355_REQUIRE(rows >= 0 && n > 0 && k > 0 && k <= 16384, MI355_ERR_INVALID, "moe_router_logits: bad shape");
   if (rows == 0) return MI355_OK;
-  hipLaunchKernelGGL(moe_router_logits_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), (size_t)4 * k * sizeof(float),
-                     (hipStream_t)stream, out, x, weight, rows, n, k);
+  hipLaunchKernelGGL(moe_router_logits_kernel, dim3((unsigned)rows), dim3(256), (size_t)k * sizeof(float), (hipStream_t)stream, out,
+                     x, weight, n, k);
   MI355_CHECK_LAUNCH("moe_router_logits");
   return MI355_OK;
 }

@@ -1452,7 +1452,7 @@ def moe_router_logits(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     _gpu(x, weight)
     assert x.dtype == torch.float32 and weight.dtype == torch.float32 and x.is_contiguous() and weight.is_contiguous()
     T, K = x.shape
-    if T > ROUTER_SKINNY_MAX_ROWS or K > 8192:
+    if T > ROUTER_SKINNY_MAX_ROWS or K > 16384:
         return linear(x, weight)
     out = torch.empty((T, weight.shape[0]), dtype=torch.float32, device=x.device)
     check(_lib_().mi355_moe_router_logits(out.data_ptr(), x.data_ptr(), weight.data_ptr(), T, weight.shape[0], K, _stream(x)),
