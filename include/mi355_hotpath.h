@@ -774,6 +774,12 @@ int mi355_sigmoid_attention(void* out, const void* q, const void* k_cache, const
 int mi355_moe_route_grouped(int32_t* ids, float* weights, const float* logits, const float* correction, int64_t tokens,
                             int num_experts, int top, int n_groups, int keep_groups, float scale, void* stream);
 int mi355_moe_block_rows(int wide);
+/* The grouped GEMM over 256-row blocks on the prefill projection kernel (mi355_linear_tiled's): every 256-row tile of the
+ * sorted rows multiplies weight[tile_expert[tile]]; row_map (null: identity) gathers the rows of x; tiles at or past
+ * *tiles_used are skipped; act 1 = erf-GELU.  Same shape conditions as mi355_linear_tiled, rows a multiple of 256. */
+int mi355_moe_grouped_linear_tiled(void* y, const void* x, int64_t x_stride, const void* w, const int32_t* row_map,
+                                   const int32_t* tile_expert, const int32_t* tiles_used, int act, int64_t rows, int64_t n,
+                                   int64_t k, int dtype, void* stream);
 int mi355_moe_router_logits(float* out, const float* x, const float* weight, int64_t rows, int n, int k, void* stream);
 int mi355_moe_align(int32_t* src_row, int32_t* rows, int32_t* tile_expert, int32_t* n_tiles, const int32_t* ids, int64_t tokens,
                     int top, int num_experts, int block, int64_t padded, void* stream);

@@ -113,6 +113,7 @@ _SIGNATURES = {
     "mi355_sigmoid_attention": (I, [P, P, P, P, P, P, P, P, P, L, P, P, L, L, L, L, L, I, I, I, I, F, I, P, L, I, I, P]),
     "mi355_moe_route_grouped": (I, [P, P, P, P, L, I, I, I, I, F, P]),
     "mi355_moe_block_rows": (I, [I]),
+    "mi355_moe_grouped_linear_tiled": (I, [P, P, L, P, P, P, P, I, L, L, L, I, P]),
     "mi355_moe_router_logits": (I, [P, P, P, L, I, I, P]),
     "mi355_moe_align": (I, [P, P, P, P, P, L, I, I, I, L, P]),
     "mi355_moe_grouped_linear": (I, [P, P, L, P, P, P, P, I, I, L, I, I, I, I, P]),

@@ -375,14 +375,15 @@ def verozen_ff_and_stream_kernels(s: dict, tokens: int) -> dict:
     ids, wts = ops.moe_route_grouped(logits, corr, top, s["groups"], s["keep"], 1.0)
     t = _timed(lambda: ops.moe_route_grouped(logits, corr, top, s["groups"], s["keep"], 1.0), 10)
     res["moe_route_grouped"] = dict(us=round(t * 1e6, 1))
-    plan = ops.moe_align(ids, E, wide_ok=True)
-    t = _timed(lambda: ops.moe_align(ids, E, wide_ok=True), 10)
+    plan = ops.moe_align(ids, E, wide_ok=True, tiled_ok=tokens > 64)
+    t = _timed(lambda: ops.moe_align(ids, E, wide_ok=True, tiled_ok=tokens > 64), 10)
     res["moe_align"] = dict(us=round(t * 1e6, 1))
     a = ops.moe_grouped_linear(h, up, plan, gather=True, gelu=True)
     t1 = _timed(lambda: ops.moe_grouped_linear(h, up, plan, gather=True, gelu=True), 5)
     t2 = _timed(lambda: ops.moe_grouped_linear(a, down, plan, gather=False, gelu=False), 5)
     fl = tokens * top * 2 * ff * D
     wbytes = E * ff * D * 2
+    res["moe_block_rows"] = plan.block
     res["moe_up_gelu"] = dict(us=round(t1 * 1e6, 1), tflops=round(fl / t1 / 1e12, 1), of_mfma_peak=round(fl / t1 / MFMA_BF16_PEAK, 3),
                               weight_gbs=round(wbytes / t1 / 1e9))
     res["moe_down"] = dict(us=round(t2 * 1e6, 1), tflops=round(fl / t2 / 1e12, 1), of_mfma_peak=round(fl / t2 / MFMA_BF16_PEAK, 3),

@@ -62,6 +62,12 @@ struct GemmTiledParams {
   int64_t kv_slot, kv_head;   // elements between consecutive slots / kv heads of the two buffers
   const void* loc;            // [M] cache slot of each row, int64 or int32
   int loc_i32;
+  // EPI 3 (grouped: every 256-row tile of x multiplies the weight matrix of the tile's own expert)
+  const int32_t* row_map;      // [M] source row of x for output row m (negative: a padding row), or null: row m itself
+  const int32_t* tile_expert;  // [mt] which of the stacked weight matrices tile tm uses
+  const int32_t* tiles_used;   // device scalar: tiles at or past it are not computed
+  int64_t w_expert_stride;     // elements between consecutive weight matrices
+  int act;                     // 1: erf-GELU on the result
 };
 
 __device__ __forceinline__ void glds16(const void* g, char* l) {
@@ -210,10 +216,14 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(GemmTiledParams p) {
   const int sup_m = st / p.snt, sup_n = st - sup_m * p.snt;
   const int tm = sup_m * 8 + (within & 7), tn = sup_n * 4 + (within >> 3);
   if (tm >= p.mt || tn >= p.nt) return;
+  if constexpr (EPI == 3) {
+    if (tm >= *p.tiles_used) return;
+  }
 
   const int T_ = (p.K * ES) >> 7;   // K tiles of 128 bytes per row
   const char* xg = (const char*)p.x;
   const char* wg = (const char*)p.w;
+  if constexpr (EPI == 3) wg += (int64_t)p.tile_expert[tm] * p.w_expert_stride * ES;
   const int ncols = EPI == 1 ? (p.N >> 1) : p.N;   // output columns
 
   // ---- per-lane source pointers of the eight load instructions a wave issues per K tile -----
@@ -239,6 +249,10 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(GemmTiledParams p) {
     for (int h = 0; h < 2; ++h) {
       int m = tm * 256 + h * 128 + rr;
       m = m < p.M ? m : p.M - 1;
+      if constexpr (EPI == 3) {
+        // gathered rows; a padding row reads row 0 (its products are stored but never read)
+        if (p.row_map != nullptr) m = max(p.row_map[m], 0);
+      }
       xs[h] = xg + ((int64_t)m * p.ldx) * ES + c * 16;
       const int rb = h * 128 + rr, wcb = rb >> 6, sl = rb & 63, ni = sl >> 4, ii = sl & 15;
       int n;
@@ -436,6 +450,12 @@ __global__ __launch_bounds__(512) void gemm_tiled_kernel(GemmTiledParams p) {
           for (int r = 0; r < 4; ++r) {
             float v0 = acc[mi][ni][r], v1 = acc[mi][2 + ni][r];
             if (FP8) { v0 = (v0 * sxm[mi]) * sw[ni * 4 + r]; v1 = (v1 * sxm[mi]) * sw[8 + ni * 4 + r]; }
+            if constexpr (EPI == 3) {
+              if (p.act == 1) {
+                v0 = 0.5f * v0 * (1.0f + erff(v0 * 0.7071067811865476f));
+                v1 = 0.5f * v1 * (1.0f + erff(v1 * 0.7071067811865476f));
+              }
+            }
             o0.v[ni * 4 + r] = from_f32<T>(v0 + bv[ni * 4 + r]);
             o1.v[ni * 4 + r] = from_f32<T>(v1 + bv[8 + ni * 4 + r]);
           }
@@ -454,13 +474,15 @@ int launch_gemm_tiled(const GemmTiledParams& p, hipStream_t st) {
   (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, GT_LDS);
   const int groups = (p.nsuper + 7) / 8;   // every XCD label gets the same number of 8 x 4 blocks
   hipLaunchKernelGGL(kern, dim3((unsigned)(groups * 8 * 32)), dim3(512), GT_LDS, st, p);
-  MI355_CHECK_LAUNCH(EPI == 2 ? "mi355_qkv_proj_rope_tiled" : FP8 ? "mi355_fp8_scaled_mm_tiled" : "mi355_linear_tiled");
+  MI355_CHECK_LAUNCH(EPI == 3 ? "mi355_moe_grouped_linear_tiled" : EPI == 2 ? "mi355_qkv_proj_rope_tiled"
+                     : FP8 ? "mi355_fp8_scaled_mm_tiled" : "mi355_linear_tiled");
   return MI355_OK;
 }
 
 void fill_tiles(GemmTiledParams& p, int64_t m, int64_t n, int epilogue) {
   p.positions = nullptr; p.cos_sin = nullptr; p.cs_f32 = 0; p.hq = p.hkv = 0;
   p.k_buffer = p.v_buffer = nullptr; p.loc = nullptr; p.loc_i32 = 0; p.kv_slot = p.kv_head = 0;
+  p.row_map = p.tile_expert = p.tiles_used = nullptr; p.w_expert_stride = 0; p.act = 0;
   const int ncols = epilogue == 1 ? (int)(n / 2) : (int)n;
   p.ldy = ncols;
   p.mt = cdiv(m, 256);
@@ -503,6 +525,26 @@ extern "C" int mi355_linear_tiled(void* y, const void* x, const void* w, const v
   if (dtype == MI355_BF16)
     return epilogue == 1 ? launch_gemm_tiled<bf16_t, 1, false>(p, st) : launch_gemm_tiled<bf16_t, 0, false>(p, st);
   return epilogue == 1 ? launch_gemm_tiled<f16_t, 1, false>(p, st) : launch_gemm_tiled<f16_t, 0, false>(p, st);
+}
+
+extern "C" int mi355_moe_grouped_linear_tiled(void* y, const void* x, int64_t x_stride, const void* w, const int32_t* row_map,
+                                              const int32_t* tile_expert, const int32_t* tiles_used, int act, int64_t rows,
+                                              int64_t n, int64_t k, int dtype, void* stream) {
+  MI355_REQUIRE(y && x && w && tile_expert && tiles_used, MI355_ERR_INVALID, "mi355_moe_grouped_linear_tiled: null pointer");
+  MI355_REQUIRE(rows > 0 && rows % 256 == 0 && mi355_linear_tiled_supported(rows, n, k, dtype, 0), MI355_ERR_UNSUPPORTED,
+                "mi355_moe_grouped_linear_tiled: needs whole 256-row tiles, a 16-bit dtype, K %% 64 == 0, K >= 128, N %% 16 == 0 "
+                "(rows=%ld n=%ld k=%ld dtype=%d)", (long)rows, (long)n, (long)k, dtype);
+  MI355_REQUIRE(x_stride >= k && x_stride % 8 == 0 && aligned16(x) && aligned16(w) && aligned16(y), MI355_ERR_INVALID,
+                "mi355_moe_grouped_linear_tiled: rows of x and the pointers must be 16-byte aligned");
+  GemmTiledParams p;
+  p.x = x; p.w = w; p.bias = nullptr; p.y = y;
+  p.x_scale = nullptr; p.w_scale = nullptr;
+  p.M = (int)rows; p.N = (int)n; p.K = (int)k;
+  p.ldx = x_stride;
+  fill_tiles(p, rows, n, 0);
+  p.row_map = row_map; p.tile_expert = tile_expert; p.tiles_used = tiles_used; p.w_expert_stride = n * k; p.act = act;
+  hipStream_t st = (hipStream_t)stream;
+  return dtype == MI355_BF16 ? launch_gemm_tiled<bf16_t, 3, false>(p, st) : launch_gemm_tiled<f16_t, 3, false>(p, st);
 }
 
 extern "C" int mi355_fp8_scaled_mm_tiled_supported(int64_t m, int64_t n, int64_t k, int out_dtype, int epilogue) {

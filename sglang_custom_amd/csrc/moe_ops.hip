@@ -471,7 +471,9 @@ int mi355_moe_route_grouped(int32_t* ids, float* weights, const float* logits, c
   return MI355_OK;
 }
 
-int mi355_moe_block_rows(int wide) { return wide ? MOE_WIDE : MOE_BLOCK; }
+constexpr int MOE_TILED = 256;     // rows of a block of the prefill projection kernel (gemm_tiled.hip)
+
+int mi355_moe_block_rows(int wide) { return wide >= 2 ? MOE_TILED : wide == 1 ? MOE_WIDE : MOE_BLOCK; }
 
 int mi355_moe_router_logits(float* out, const float* x, const float* weight, int64_t rows, int n, int k, void* stream) {
   MI355_REQUIRE(out && x && weight, MI355_ERR_INVALID, "moe_router_logits: null pointer");
@@ -485,7 +487,8 @@ int mi355_moe_router_logits(float* out, const float* x, const float* weight, int
 
 int mi355_moe_align(int32_t* src_row, int32_t* rows, int32_t* tile_expert, int32_t* n_tiles, const int32_t* ids, int64_t tokens,
                     int top, int num_experts, int block, int64_t padded, void* stream) {
-  MI355_REQUIRE(block == MOE_BLOCK || block == MOE_WIDE, MI355_ERR_INVALID, "moe_align: blocks of %d or %d rows", MOE_BLOCK, MOE_WIDE);
+  MI355_REQUIRE(block == MOE_BLOCK || block == MOE_WIDE || block == MOE_TILED, MI355_ERR_INVALID, "moe_align: blocks of %d, %d or %d rows",
+                MOE_BLOCK, MOE_WIDE, MOE_TILED);
   MI355_REQUIRE(src_row && rows && tile_expert && n_tiles && ids, MI355_ERR_INVALID, "moe_align: null pointer");
   MI355_REQUIRE(tokens >= 0 && top > 0 && num_experts > 0 && num_experts <= 4096, MI355_ERR_INVALID, "moe_align: bad shape");
   MI355_REQUIRE(padded % block == 0 && padded >= tokens * top + (int64_t)std::min<int64_t>(num_experts, tokens * top) * (block - 1),
@@ -502,6 +505,9 @@ int mi355_moe_grouped_linear(void* out, const void* in, int64_t in_stride, const
                              const int32_t* tile_expert, const int32_t* n_tiles, int gather, int gelu, int64_t padded, int block,
                              int n, int k, int dtype, void* stream) {
   MI355_REQUIRE(out && in && weight && src_row && tile_expert && n_tiles, MI355_ERR_INVALID, "moe_grouped_linear: null pointer");
+  if (block == MOE_TILED)
+    return mi355_moe_grouped_linear_tiled(out, in, in_stride, weight, gather ? src_row : nullptr, tile_expert, n_tiles, gelu ? 1 : 0,
+                                          padded, n, k, dtype, stream);
   MI355_REQUIRE(block == MOE_BLOCK || block == MOE_WIDE, MI355_ERR_INVALID, "moe_grouped_linear: blocks of %d or %d rows", MOE_BLOCK,
                 MOE_WIDE);
   MI355_REQUIRE(padded >= 0 && padded % block == 0 && n > 0 && k > 0 && in_stride >= k && padded / block <= 65535,

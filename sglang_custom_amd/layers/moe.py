@@ -47,8 +47,11 @@ class GroupedExperts(nn.Module):
         """h [T, D], expert_ids int32 [T, top] -> (y [P, D], rows int32 [T, top]): y[rows[t, j]] is the output of token
         t's j-th expert; P >= T * top counts the padding of the experts' blocks."""
         ops = get_ops()
-        plan = ops.moe_align(expert_ids, self.num_experts,
-                             wide_ok=h.dtype != torch.float32 and self.hidden % 8 == 0 and self.ff % 8 == 0)
+        sixteen = h.dtype != torch.float32
+        plan = ops.moe_align(expert_ids, self.num_experts, wide_ok=sixteen and self.hidden % 8 == 0 and self.ff % 8 == 0,
+                             tiled_ok=sixteen and h.shape[0] > 64 and h.stride(0) % 8 == 0
+                             and ops.linear_tiled_supported(256, self.ff, self.hidden, h.dtype)
+                             and ops.linear_tiled_supported(256, self.hidden, self.ff, h.dtype))
         a = ops.moe_grouped_linear(h, self.w_up.data, plan, gather=True, gelu=True)
         y = ops.moe_grouped_linear(a, self.w_down.data, plan, gather=False, gelu=False)
         return y, plan.rows

@@ -1460,14 +1460,15 @@ def moe_router_logits(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def moe_align(expert_ids: torch.Tensor, num_experts: int, wide_ok: bool = False) -> MoePlan:
-    """wide_ok: the grouped GEMMs that follow can take blocks of 128 rows (16-bit operands, 16-byte rows); they are used
-    when the experts have at least two such blocks' worth of rows on average."""
+def moe_align(expert_ids: torch.Tensor, num_experts: int, wide_ok: bool = False, tiled_ok: bool = False) -> MoePlan:
+    """wide_ok: the grouped GEMMs that follow can take blocks of 128 rows (16-bit operands, 16-byte rows); tiled_ok: they
+    can run on the prefill projection kernel over blocks of 256 rows (linear_tiled_supported for both of them).  The
+    larger blocks are used when the experts have at least two of them worth of rows on average."""
     _gpu(expert_ids)
     T, top = expert_ids.shape
     assert expert_ids.dtype == torch.int32 and expert_ids.is_contiguous()
-    wide = bool(wide_ok) and T * top >= 256 * num_experts
-    block = int(_lib_().mi355_moe_block_rows(int(wide)))
+    wide = 2 if (tiled_ok and T * top >= 512 * num_experts) else 1 if ((wide_ok or tiled_ok) and T * top >= 256 * num_experts) else 0
+    block = int(_lib_().mi355_moe_block_rows(wide))
     pairs = T * top
     padded = (pairs + min(num_experts, pairs) * (block - 1) + block - 1) // block * block
     dev = expert_ids.device

@@ -460,7 +460,11 @@ def moe_router_logits(x, weight):
     return F.linear(x, weight)
 
 
-def moe_align(expert_ids, num_experts, wide_ok=False, block=4):
+def linear_tiled_supported(m, n, k, dtype, silu_mul=False):
+    return False
+
+
+def moe_align(expert_ids, num_experts, wide_ok=False, tiled_ok=False, block=4):
     T, top = expert_ids.shape
     flat = expert_ids.reshape(-1).tolist()
     src, tiles = [], []

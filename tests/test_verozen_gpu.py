@@ -102,7 +102,14 @@ def test_experts_over_sorted_blocks(dtype, T, D, ff, E, top):
 def test_experts_over_wide_blocks(D, ff):
     """Enough rows per expert for the 128-row blocks of the prefill-sized kernel: K tiles with a tail (200, 72), one idle
     expert, column counts that are no multiple of the tile."""
-    cases.check_experts(ops(), DEV, torch.bfloat16, T=1100, D=D, ff=ff, E=4, top=2, wide_ok=True)
+    cases.check_experts(ops(), DEV, torch.bfloat16, T=1100, D=D, ff=ff, E=4, top=2, wide_ok=True, block=128)
+
+
+@pytest.mark.parametrize("D,ff", [(128, 192), (256, 128)])
+def test_experts_over_blocks_of_the_prefill_projection_kernel(D, ff):
+    """Blocks of 256 rows on the package's prefill GEMM kernel with per-block weights, gathered rows and the activation in
+    its epilogue: widths that are multiples of 64, one idle expert, a partly filled last block per expert."""
+    cases.check_experts(ops(), DEV, torch.bfloat16, T=2300, D=D, ff=ff, E=4, top=2, tiled_ok=True, block=256)
 
 
 def test_router_logits_few_rows_and_many():

@@ -298,7 +298,7 @@ def check_router_logits(ops, device, T, D=200, E=12):
     _close(ops.moe_router_logits(x.to(device), w.to(device)), x.double() @ w.double().T, 2e-6, "router logits in fp32")
 
 
-def check_experts(ops, device, dtype, T=37, D=48, ff=40, E=5, top=2, wide_ok=False):
+def check_experts(ops, device, dtype, T=37, D=48, ff=40, E=5, top=2, wide_ok=False, tiled_ok=False, block=None):
     g = torch.Generator().manual_seed(6)
     h = _bf(torch.randn(T, D, generator=g))
     up = _bf(torch.randn(E, ff, D, generator=g) * D ** -0.5)
@@ -309,7 +309,8 @@ def check_experts(ops, device, dtype, T=37, D=48, ff=40, E=5, top=2, wide_ok=Fal
         for t in range(T):
             if -1 in ids[t].tolist():
                 ids[t][ids[t] == -1] = [e for e in range(E - 1) if e not in ids[t].tolist()][0]
-    plan = ops.moe_align(ids.to(device), E, wide_ok=wide_ok)
+    plan = ops.moe_align(ids.to(device), E, wide_ok=wide_ok, tiled_ok=tiled_ok)
+    assert block is None or plan.block == block
     a = ops.moe_grouped_linear(h.to(dtype).to(device), up.to(dtype).to(device), plan, gather=True, gelu=True)
     y = ops.moe_grouped_linear(a, down.to(dtype).to(device), plan, gather=False, gelu=False)
     rows = plan.rows.cpu().long()
