@@ -56,8 +56,10 @@ __global__ __launch_bounds__(256) void sigmoid_attention_valu_kernel(SgArgs a) {
   const int chunks = (rep + a.heads_per_tile - 1) / a.heads_per_tile;
   const int g = blockIdx.y / chunks, hc = blockIdx.y - g * chunks;
   const int split = blockIdx.z;
-  const int64_t t0 = a.blocks != nullptr ? a.blocks[2 * blockIdx.x] : blockIdx.x;
-  const int nt = a.blocks != nullptr ? a.blocks[2 * blockIdx.x + 1] : 1;
+  // runs come in token order, so a sequence's later (longer) runs are listed last: take them first
+  const unsigned bx = gridDim.x - 1 - blockIdx.x;
+  const int64_t t0 = a.blocks != nullptr ? a.blocks[2 * bx] : bx;
+  const int nt = a.blocks != nullptr ? a.blocks[2 * bx + 1] : 1;
   const int b = a.tok_req != nullptr ? a.tok_req[t0] : (int)t0;
   const int32_t* table = a.req_to_token + a.req_pool_indices[b] * a.req_to_token_stride;
   const int h0 = g * rep + hc * a.heads_per_tile;
@@ -176,8 +178,10 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
   const int chunks = (rep + HR - 1) / HR;
   const int g = blockIdx.y / chunks, hc = blockIdx.y - g * chunks;
   const int split = blockIdx.z;
-  const int64_t t0 = a.blocks != nullptr ? a.blocks[2 * blockIdx.x] : blockIdx.x;
-  const int nt = a.blocks != nullptr ? a.blocks[2 * blockIdx.x + 1] : 1;
+  // runs come in token order, so a sequence's later (longer) runs are listed last: take them first
+  const unsigned bx = gridDim.x - 1 - blockIdx.x;
+  const int64_t t0 = a.blocks != nullptr ? a.blocks[2 * bx] : bx;
+  const int nt = a.blocks != nullptr ? a.blocks[2 * bx + 1] : 1;
   const int b = a.tok_req != nullptr ? a.tok_req[t0] : (int)t0;
   const int32_t* table = a.req_to_token + a.req_pool_indices[b] * a.req_to_token_stride;
   const int h0 = g * rep + hc * HR;
@@ -197,7 +201,7 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
 #pragma unroll
       for (int x = 0; x < 8; ++x) val.v[x] = from_f32<T>(0.f);
     }
-    stvec<T, 8>(Qs + r * qld + ch * 8, val);
+    lds_store16(Qs + r * qld + ch * 8, val);
   }
   if (tid < SGM_ROWS) {
     const int tl = tid / HR, hl = tid - tl * HR;
@@ -220,20 +224,34 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
   const T* vc = (const T*)a.v_cache;
   using Frag = typename Mfma<T>::frag;
   Vec<T, 8> kreg[SGM_MAXC], vreg[SGM_MAXC];
-  // every load is unconditional (a load under a branch is waited for at the branch's end, one latency per load): chunk
-  // numbers past the tile's last one are clamped to it -- all lanes then read one address -- and never stored
-  auto request = [&](int tile) {
+  // Every load is unconditional (a load under a branch is waited for at the branch's end, one latency per load): chunk
+  // numbers past the tile's last one are clamped to it -- all lanes then read one address -- and never stored.  The cache
+  // slots of a tile's keys are read from the request table one tile before the rows themselves are requested, so that
+  // a request does not start with a wait for its own addresses.
+  int64_t ksrc[SGM_MAXC], vsrc[SGM_MAXC];
+  auto load_slots = [&](int tile) {
     const int j0 = tile * SG_KT;
 #pragma unroll
     for (int u = 0; u < SGM_MAXC; ++u) {
       const int ek = min(tid + 256 * u, SG_KT * dch - 1), ev = min(tid + 256 * u, SG_KT * vch - 1);
       const int kk = ek / dch, kv = ev / vch;
       // keys past the run's last one are masked below; any valid row will do
-      kreg[u] = ldvec<T, 8>(kc + ((int64_t)table[min(j0 + kk, last)] * a.kv_heads + g) * d + (ek - kk * dch) * 8);
-      vreg[u] = ldvec<T, 8>(vc + ((int64_t)table[min(j0 + kv, last)] * a.kv_heads + g) * dv + (ev - kv * vch) * 8);
+      ksrc[u] = ((int64_t)table[min(j0 + kk, last)] * a.kv_heads + g) * d + (ek - kk * dch) * 8;
+      vsrc[u] = ((int64_t)table[min(j0 + kv, last)] * a.kv_heads + g) * dv + (ev - kv * vch) * 8;
     }
   };
-  if (tile_lo < tile_hi) request(tile_lo);
+  auto request = [&]() {
+#pragma unroll
+    for (int u = 0; u < SGM_MAXC; ++u) {
+      kreg[u] = ldvec<T, 8>(kc + ksrc[u]);
+      vreg[u] = ldvec<T, 8>(vc + vsrc[u]);
+    }
+  };
+  if (tile_lo < tile_hi) {
+    load_slots(tile_lo);
+    request();
+    load_slots(tile_lo + 1);
+  }
   for (int tile = tile_lo; tile < tile_hi; ++tile) {
     const int j0 = tile * SG_KT;
     __syncthreads();                             // the last tile's readers are done (and, the first time, Qs is written)
@@ -242,21 +260,24 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
       const int e = tid + 256 * u;
       if (e < SG_KT * dch) {
         const int kk = e / dch, ch = e - kk * dch;
-        stvec<T, 8>(Ks + kk * qld + ch * 8, kreg[u]);
+        lds_store16(Ks + kk * qld + ch * 8, kreg[u]);
       }
       if (e < SG_KT * vch) {
         const int kk = e / vch, ch = e - kk * vch;
-        stvec<T, 8>(Vs + kk * vld + ch * 8, vreg[u]);
+        lds_store16(Vs + kk * vld + ch * 8, vreg[u]);
       }
     }
     __syncthreads();
-    if (tile + 1 < tile_hi) request(tile + 1);   // in flight during this tile's products
+    if (tile + 1 < tile_hi) {                    // in flight during this tile's products
+      request();
+      load_slots(tile + 2);
+    }
     if (16 * wv < live_rows) {
       f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
       for (int c = 0; c < d; c += 32) {
-        const Frag af = *reinterpret_cast<const Frag*>(Qs + (16 * wv + li) * qld + c + 8 * lg);
-        const Frag b0 = *reinterpret_cast<const Frag*>(Ks + li * qld + c + 8 * lg);
-        const Frag b1 = *reinterpret_cast<const Frag*>(Ks + (16 + li) * qld + c + 8 * lg);
+        const Frag af = lds_load16<Frag>(Qs + (16 * wv + li) * qld + c + 8 * lg);
+        const Frag b0 = lds_load16<Frag>(Ks + li * qld + c + 8 * lg);
+        const Frag b1 = lds_load16<Frag>(Ks + (16 + li) * qld + c + 8 * lg);
         s0 = Mfma<T>::run(af, b0, s0);
         s1 = Mfma<T>::run(af, b1, s1);
       }
@@ -266,8 +287,8 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
         const int r = 16 * wv + 4 * lg + x;
         const int rp = row_pos[r];
         const float m = row_mul[r], ad = row_add[r];
-        Ps[r * pld + li] = from_f32<T>(j0 + li <= rp ? sg_sigmoid(s0[x] * m + ad) : 0.f);
-        Ps[r * pld + 16 + li] = from_f32<T>(j0 + 16 + li <= rp ? sg_sigmoid(s1[x] * m + ad) : 0.f);
+        lds_store2(Ps + r * pld + li, from_f32<T>(j0 + li <= rp ? sg_sigmoid(s0[x] * m + ad) : 0.f));
+        lds_store2(Ps + r * pld + 16 + li, from_f32<T>(j0 + 16 + li <= rp ? sg_sigmoid(s1[x] * m + ad) : 0.f));
       }
     }
     __syncthreads();
@@ -285,7 +306,7 @@ __global__ __launch_bounds__(256) void sigmoid_attention_mfma_kernel(SgArgs a) {
 #pragma unroll
       for (int rt = 0; rt < 4; ++rt) {
         if (16 * rt < live_rows) {
-          const Frag pa = *reinterpret_cast<const Frag*>(Ps + (16 * rt + li) * pld + 8 * lg);
+          const Frag pa = lds_load16<Frag>(Ps + (16 * rt + li) * pld + 8 * lg);
 #pragma unroll
           for (int c = 0; c < CT; ++c) {
             if (CT * wv + c < nblk) {

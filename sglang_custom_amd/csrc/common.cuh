@@ -54,6 +54,23 @@ __device__ __forceinline__ uint2 ld8_nt(const void* p) {
 template <typename T, int N> __device__ __forceinline__ void stvec(T* p, const Vec<T, N>& x) {
   *reinterpret_cast<Vec<T, N>*>(p) = x;
 }
+// Loads and stores that are LDS instructions by construction.  A pointer into a __shared__ array that has passed through
+// pointer variables or helper functions may reach the backend as a generic pointer; the access is then a FLAT instruction,
+// which takes the vector-memory path, counts on vmcnt in order with the global loads in flight (a wait for it waits for
+// every prefetch issued before it) and is several times slower than a ds_read / ds_write.
+typedef unsigned lds_u32x4 __attribute__((ext_vector_type(4)));
+template <typename V> __device__ __forceinline__ V lds_load16(const void* p) {
+  static_assert(sizeof(V) == 16, "16-byte values");
+  return __builtin_bit_cast(V, *((const __attribute__((address_space(3))) lds_u32x4*)p));
+}
+template <typename V> __device__ __forceinline__ void lds_store16(void* p, const V& v) {
+  static_assert(sizeof(V) == 16, "16-byte values");
+  *((__attribute__((address_space(3))) lds_u32x4*)p) = __builtin_bit_cast(lds_u32x4, v);
+}
+template <typename V> __device__ __forceinline__ void lds_store2(void* p, const V& v) {
+  static_assert(sizeof(V) == 2, "2-byte values");
+  *((__attribute__((address_space(3))) unsigned short*)p) = __builtin_bit_cast(unsigned short, v);
+}
 // Elements per 16-byte access.
 template <typename T> struct V16 { static constexpr int n = 16 / sizeof(T); };
 

@@ -355,8 +355,8 @@ __global__ __launch_bounds__(256) void moe_grouped_linear_wide_kernel(T* __restr
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int c = tid + 256 * u, r = c >> 3, piece = c & 7;
-      stvec<T, 8>(As + r * MOE_WLD + piece * 8, areg[u]);
-      stvec<T, 8>(Bs + r * MOE_WLD + piece * 8, breg[u]);
+      lds_store16(As + r * MOE_WLD + piece * 8, areg[u]);
+      lds_store16(Bs + r * MOE_WLD + piece * 8, breg[u]);
     }
     __syncthreads();
     if (k0 + MOE_WK < K) request(k0 + MOE_WK);
@@ -365,8 +365,8 @@ __global__ __launch_bounds__(256) void moe_grouped_linear_wide_kernel(T* __restr
       Frag af[4], bf[4];
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
-        af[x] = *reinterpret_cast<const Frag*>(As + (wm * 64 + x * 16 + li) * MOE_WLD + kk + 8 * lg);
-        bf[x] = *reinterpret_cast<const Frag*>(Bs + (wn * 64 + x * 16 + li) * MOE_WLD + kk + 8 * lg);
+        af[x] = lds_load16<Frag>(As + (wm * 64 + x * 16 + li) * MOE_WLD + kk + 8 * lg);
+        bf[x] = lds_load16<Frag>(Bs + (wn * 64 + x * 16 + li) * MOE_WLD + kk + 8 * lg);
       }
 #pragma unroll
       for (int x = 0; x < 4; ++x)
