@@ -236,29 +236,29 @@ VEROZEN_SIZES = {
                    keep=2, ff=2048, layers=4, vocab=32768, side=64, norm_groups=8, gate_rank=64),
     "vz4096": dict(width=4096, heads=32, kv_heads=8, dim=128, rec_heads=32, rec_dim=64, rec_vdim=128, experts=64, top=8, groups=8,
                    keep=4, ff=1536, layers=4, vocab=32768, side=64, norm_groups=8, gate_rank=64),
-    "vztiny": dict(width=256, heads=8, kv_heads=2, dim=64, rec_heads=4, rec_dim=32, rec_vdim=64, experts=8, top=2, groups=4, keep=2,
-                   ff=128, layers=3, vocab=2048, side=16, norm_groups=4, gate_rank=16),
+    "vztiny": dict(width=320, heads=8, kv_heads=2, dim=64, rec_heads=4, rec_dim=32, rec_vdim=64, experts=12, top=2, groups=3, keep=2,
+                   ff=128, layers=3, vocab=2048, side=8, norm_groups=5, gate_rank=24),
 }
 
 
 def verozen_config(s: dict) -> dict:
     mlp = dict(kind="moe", expert=dict(ff=s["ff"]),
                router=dict(experts=s["experts"], top=s["top"], scale=1.0, groups=dict(count=s["groups"], keep=s["keep"])))
-    gla = dict(type="gla", mixer=dict(heads=s["rec_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"], tau=16.0, gate_rank=s["gate_rank"]), mlp=mlp)
+    gla = dict(type="gla", mixer=dict(heads=s["rec_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"], tau=8.0, gate_rank=s["gate_rank"]), mlp=mlp)
     att = dict(type="attention", mixer=dict(heads=s["heads"], kv_heads=s["kv_heads"], dim=s["dim"], vdim=s["dim"], scale=s["dim"] ** -0.5,
-                                            rot=dict(base=500000.0, dims=s["dim"] // 2)), mlp=mlp)
+                                            rot=dict(base=10000.0, dims=s["dim"] // 2)), mlp=mlp)
     ret = dict(type="retention", mixer=dict(heads=s["rec_heads"], dim=s["rec_dim"], vdim=s["rec_vdim"],
-                                            decay=[1.0 - 2.0 ** (-5 - (i % 6)) for i in range(s["rec_heads"])],
-                                            rot=dict(base=1000000.0, dims=s["rec_dim"])), mlp=mlp)
+                                            decay=[0.9 + 0.0123 * (i % 8) for i in range(s["rec_heads"])],
+                                            rot=dict(base=100000.0, dims=s["rec_dim"])), mlp=mlp)
     order = [gla, att, ret, gla]
-    return dict(architecture="Verozen", vocab=s["vocab"], width=s["width"], postln_alpha=3.0, norm=dict(eps=1e-5, groups=s["norm_groups"]),
+    return dict(architecture="Verozen", vocab=s["vocab"], width=s["width"], postln_alpha=2.0, norm=dict(eps=1e-6, groups=s["norm_groups"]),
                 token_side=dict(dim=s["side"]), layers=[order[i % 4] for i in range(s["layers"])])
 
 
 def llama_config(s: dict, dtype: str) -> dict:
     return dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=s["width"], num_hidden_layers=s["layers"],
                 num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"], head_dim=s["dim"],
-                intermediate_size=s["ff"] * s["top"], vocab_size=s["vocab"], rms_norm_eps=1e-5, rope_theta=500000.0,
+                intermediate_size=s["ff"] * s["top"], vocab_size=s["vocab"], rms_norm_eps=1e-6, rope_theta=10000.0,
                 max_position_embeddings=16384, rope_scaling=None, tie_word_embeddings=False, torch_dtype=dtype, hidden_act="silu",
                 attention_bias=False, mlp_bias=False)
 
@@ -334,7 +334,7 @@ def verozen_mixer_kernels(s: dict, bs: int, ctx: int, prefill_bs: int, prefill_l
         z = torch.randn(bs, RH * dk, device=dev, generator=g) if gated else None
         hd = None if gated else torch.full((RH,), 0.99, device=dev)
         posd = torch.full((bs,), ctx, device=dev, dtype=torch.int64)
-        t = _timed(lambda: ops.linear_recurrence(qd, kd, vd, od, state, r2s, rpi, posd, 1.0, gate_logits=z, tau=16.0, head_decay=hd), 20)
+        t = _timed(lambda: ops.linear_recurrence(qd, kd, vd, od, state, r2s, rpi, posd, 1.0, gate_logits=z, tau=8.0, head_decay=hd), 20)
         b = bs * RH * dk * dv * 4 * 2
         res[f"verozen_{name}_decode_recurrence"] = dict(us=round(t * 1e6, 1), gbs=round(b / t / 1e9), of_hbm_peak=round(b / t / HBM_PEAK, 3))
         qd = torch.randn(T, RH, dk, device=dev, generator=g).to(qk_dt)
@@ -345,7 +345,7 @@ def verozen_mixer_kernels(s: dict, bs: int, ctx: int, prefill_bs: int, prefill_l
         ss = torch.arange(0, T, prefill_len, device=dev, dtype=torch.int32)
         sl = torch.full((prefill_bs,), prefill_len, device=dev, dtype=torch.int32)
         t = _timed(lambda: ops.linear_recurrence(qd, kd, vd, od, state, r2s, torch.arange(prefill_bs, device=dev), posp, 1.0,
-                                                 gate_logits=z, tau=16.0, head_decay=hd, tok_req=tok_req, seg_start=ss, seg_len=sl), 3)
+                                                 gate_logits=z, tau=8.0, head_decay=hd, tok_req=tok_req, seg_start=ss, seg_len=sl), 3)
         fl = T * RH * dk * dv * 6
         res[f"verozen_{name}_prefill_recurrence"] = dict(ms=round(t * 1e3, 3), vector_tflops=round(fl / t / 1e12, 2),
                                                           tokens_per_s_per_sequence=round(prefill_len / t))

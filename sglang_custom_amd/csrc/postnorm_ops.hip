@@ -20,30 +20,70 @@ __device__ __forceinline__ float pn_gelu_tanh(float z) {
 }
 __device__ __forceinline__ float pn_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 
+// Eight consecutive features of a row of T: one 16-byte load for 16-bit types, two for fp32.
+template <typename T> __device__ __forceinline__ Vec<T, 8> ld_row8(const T* p) {
+  if constexpr (sizeof(T) == 2) {
+    return ldvec<T, 8>(p);
+  } else {
+    Vec<T, 8> r;
+    const Vec<T, 4> a = ldvec<T, 4>(p), b = ldvec<T, 4>(p + 4);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { r.v[k] = a.v[k]; r.v[4 + k] = b.v[k]; }
+    return r;
+  }
+}
+
 // One workgroup per token.  sm holds the row (D floats) and then one 1/rms per group.
 template <typename T>
 __global__ __launch_bounds__(256) void scaled_add_group_rmsnorm_kernel(
     float* x_out, T* __restrict__ h_out, const float* x, const T* __restrict__ branch,
     int64_t branch_stride, const int32_t* __restrict__ rows, const float* __restrict__ coef, int n_branch, float alpha,
-    const T* __restrict__ w, int64_t D, int groups, float eps) {
+    const T* __restrict__ w, int64_t D, int groups, float eps, bool vec8) {
   extern __shared__ __attribute__((aligned(16))) float sm[];
   __shared__ float red[16];
   float* row = sm;
   float* inv = sm + D;
   const int64_t t = blockIdx.x;
-  for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
-    float s = alpha * x[t * D + i];
-    if (branch != nullptr) {
-      if (rows == nullptr) {
-        s += to_f32(branch[t * branch_stride + i]);
-      } else {
-        float b = 0.f;
-        for (int j = 0; j < n_branch; ++j)      // fixed order: the sum does not depend on where the rows lie
-          b += coef[t * n_branch + j] * to_f32(branch[(int64_t)rows[t * n_branch + j] * branch_stride + i]);
-        s += b;
+  if (vec8) {
+    // eight features per thread and access: 16-byte loads of the branch rows, two of the fp32 row
+    for (int64_t i = 8 * threadIdx.x; i < D; i += 8 * blockDim.x) {
+      const float4 x0 = *reinterpret_cast<const float4*>(x + t * D + i), x1 = *reinterpret_cast<const float4*>(x + t * D + i + 4);
+      float s[8] = {alpha * x0.x, alpha * x0.y, alpha * x0.z, alpha * x0.w, alpha * x1.x, alpha * x1.y, alpha * x1.z, alpha * x1.w};
+      if (branch != nullptr) {
+        if (rows == nullptr) {
+          const Vec<T, 8> b = ld_row8<T>(branch + t * branch_stride + i);
+#pragma unroll
+          for (int k = 0; k < 8; ++k) s[k] += to_f32(b.v[k]);
+        } else {
+          float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          for (int j = 0; j < n_branch; ++j) {      // fixed order: the sum does not depend on where the rows lie
+            const float c = coef[t * n_branch + j];
+            const Vec<T, 8> b = ld_row8<T>(branch + (int64_t)rows[t * n_branch + j] * branch_stride + i);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc[k] += c * to_f32(b.v[k]);
+          }
+#pragma unroll
+          for (int k = 0; k < 8; ++k) s[k] += acc[k];
+        }
       }
+#pragma unroll
+      for (int k = 0; k < 8; ++k) row[i + k] = s[k];
     }
-    row[i] = s;
+  } else {
+    for (int64_t i = threadIdx.x; i < D; i += blockDim.x) {
+      float s = alpha * x[t * D + i];
+      if (branch != nullptr) {
+        if (rows == nullptr) {
+          s += to_f32(branch[t * branch_stride + i]);
+        } else {
+          float b = 0.f;
+          for (int j = 0; j < n_branch; ++j)      // fixed order: the sum does not depend on where the rows lie
+            b += coef[t * n_branch + j] * to_f32(branch[(int64_t)rows[t * n_branch + j] * branch_stride + i]);
+          s += b;
+        }
+      }
+      row[i] = s;
+    }
   }
   __syncthreads();
   const int64_t gs = D / groups;
@@ -202,10 +242,11 @@ int mi355_scaled_add_group_rmsnorm(float* x_out, void* h_out, const float* x, co
                 "scaled_add_group_rmsnorm: rows, coef and the branch come together");
   if (tokens == 0) return MI355_OK;
   const size_t lds = (size_t)(hidden + groups) * sizeof(float);
+  const bool vec8 = hidden % 8 == 0 && aligned16(x) && (branch == nullptr || (branch_stride % 8 == 0 && aligned16(branch)));
   MI355_DISPATCH_DTYPE(dtype, "scaled_add_group_rmsnorm", {
     hipLaunchKernelGGL((scaled_add_group_rmsnorm_kernel<T>), dim3((unsigned)tokens), dim3(256), lds, (hipStream_t)stream, x_out,
                        (T*)h_out, x, (const T*)branch, branch_stride, rows, coef, n_branch, alpha, (const T*)weight, hidden,
-                       groups, eps);
+                       groups, eps, vec8);
   });
   MI355_CHECK_LAUNCH("scaled_add_group_rmsnorm");
   return MI355_OK;
