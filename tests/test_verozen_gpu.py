@@ -67,10 +67,12 @@ def test_recurrence_far_keys_first_tokens_and_slots(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,G,d", [(4, 2, 32), (8, 1, 64), (3, 3, 24), (32, 1, 32), (6, 2, 128), (1, 1, 8)])
+@pytest.mark.parametrize("H,G,d", [(4, 2, 32), (8, 1, 64), (3, 3, 24), (32, 1, 32), (6, 2, 128), (1, 1, 8), (4, 2, 96), (2, 1, 160),
+                                   (128, 1, 32), (2, 2, 256)])
 def test_sigmoid_attention_whole_cut_and_decoded(dtype, H, G, d):
-    """Widths of 32 and more run on the matrix cores in bf16, 24 and 8 on the vector ALU; 32 heads on one key head is two
-    workgroups per token."""
+    """Multiples of 32 run on the matrix cores in bf16 (96 and 160: tiles whose chunk counts are no power of two, column
+    tiles that do not fill the four waves; 256: the widest), 24 and 8 on the vector ALU; 128 heads on one key head is two
+    workgroups per run on the matrix cores, eight on the vector ALU."""
     for cuts, tail, page, splits in (((150,), 0, 1, 1), ((63, 2, 1, 84), 0, 64, 1), ((140,) + (1,) * 10, 10, 16, 1),
                                      ((146, 1, 1, 1, 1), 4, 1, 3)):
         cases.check_sigmoid_attention(ops(), DEV, dtype, H=H, G=G, d=d, cuts=cuts, decode_tail=tail, page=page, splits=splits)
